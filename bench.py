@@ -1,0 +1,150 @@
+"""Benchmark of the VQ-attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One step = one seqlen_q = 1 VQ-attention call (lookup table + streaming kernel + split merge) over the decode
+configuration: batch 16, 32 heads, head_dim 128, 32768 keys, 4 codebooks x 256 codewords, bf16, inputs resident in
+HBM.  Prints ONE JSON line.  `value` is the achieved HBM rate of the whole step: algorithmic bytes (codes + V +
+codebooks + q + out, each touched once) divided by the step time.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
+
+
+def cpu_baseline(case, units=32, repeats=3):
+    """The fp32 PyTorch oracle timed on the host cores over `units` (batch, head) problems of the same workload.
+
+    Returns the equivalent HBM rate (algorithmic bytes of the sampled units / time) so it is comparable with `value`.
+    """
+    import torch
+
+    import oracle
+
+    B, H = case.q.shape[:2]
+    units = min(units, B * H)
+    idx = [(u * 7) % (B * H) for u in range(units)]  # spread over batches and heads
+    sample = []
+    for u in idx:
+        b, h = divmod(u, H)
+        sample.append((case.q[b:b + 1, h:h + 1].cpu(), case.codes[b:b + 1, h:h + 1].cpu(),
+                       case.codebooks[h:h + 1].cpu(), case.v[b:b + 1, h:h + 1].cpu()))
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    times = []
+    for r in range(repeats + 1):
+        t0 = time.perf_counter()
+        for q, c, cb, v in sample:
+            oracle.attn_vq_decode(q, c, cb, v, case.softmax_scale)
+        times.append(time.perf_counter() - t0)
+    t = sorted(times[1:])[len(times[1:]) // 2]
+    e = case.q.element_size()
+    D = case.q.shape[-1]
+    N, M = case.codes.shape[2], case.codes.shape[3]
+    bytes_per_unit = N * M + N * D * e + case.codebooks[0].numel() * e + 2 * D * e
+    return {
+        "value": round(units * bytes_per_unit / t / 1e9, 3),
+        "unit": "GB/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"{units} of {B * H} (batch, head) units of the same workload, fp32 PyTorch oracle, "
+                  f"median of {repeats} runs, {t * 1e3:.1f} ms",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU only: the VQ-attention path shards over (batch, head) with no "
+                 "communication, and this build runs on single-GPU boxes; run with --gpus 1")
+
+    import torch
+
+    from vqtree_amd import _lib
+    from vqtree_amd.ops.attn_vq import attn_vq_decode
+    from vqtree_amd.synthetic import decode_c2
+
+    _lib.load()  # fail loudly if the HIP library is missing
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    case = decode_c2(dev)
+    B, H, N, M = case.codes.shape
+    D = case.q.shape[-1]
+    K = case.codebooks.shape[2]
+
+    def step():
+        return attn_vq_decode(case.q, case.codes, case.codebooks, case.v, softmax_scale=case.softmax_scale)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    # HIP events on the stream the kernels run on (torch's current stream is the one handed to the library)
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        starts[i].record()
+        step()
+        ends[i].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ev_ms = [s.elapsed_time(e) for s, e in zip(starts, ends)]
+    ms_per_step = wall * 1e3 / args.steps
+    kern_ms = sum(ev_ms) / len(ev_ms)
+
+    alg_bytes = case.algorithmic_bytes
+    value = alg_bytes / (ms_per_step * 1e-3) / 1e9
+    achieved = alg_bytes / (kern_ms * 1e-3) / 1e9
+    result = {
+        "metric": "VQ-attn decode HBM GB/s @32k (us/step in us_per_step)",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "us_per_step": round(ms_per_step * 1e3, 1),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": f"VQ-attention decode seqlen_q=1: batch {B}, {H} heads, head_dim {D}, KV context {N}, "
+                        f"{M} codebooks x {K} codewords, uint8 codes, bf16 q/V/codebooks, no mask",
+            "algorithmic_bytes_per_step": alg_bytes,
+        },
+        "roofline": {
+            "bound": "hbm",
+            "achieved": round(achieved, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBPS, 4),
+            "traffic": None,
+            "kernel": "vqa::decode::main_kernel<bf16,128,4>",
+            "duration_us": round(kern_ms * 1e3, 1),
+            "duration_covers": "HIP events around the whole call (lookup-table + streaming + merge kernels); the "
+                               "streaming kernel is >98% of it",
+        },
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(case)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,77 @@
+"""CPU-side checks of the C-ABI library: it loads, exports every symbol include/vqattn.h declares, and its
+host-only entry points (no kernel launch) behave."""
+import os
+import re
+
+import pytest
+
+from vqtree_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "vqattn.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(vqa_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported_and_bound(lib):
+    declared = _declared_symbols()
+    assert declared, "no declarations parsed"
+    for name in declared:
+        assert hasattr(lib, name), f"{name} declared in include/vqattn.h but not exported"
+        assert name in _lib.SIGNATURES, f"{name} has no ctypes signature in vqtree_amd/_lib.py"
+    assert sorted(_lib.SIGNATURES) == declared
+
+
+def test_version_and_error_strings(lib):
+    assert lib.vqa_version() >= 100
+    assert lib.vqa_strerror(0) == b"ok"
+    seen = set()
+    for code in range(-8, 0):
+        msg = lib.vqa_strerror(code)
+        assert msg and msg != b"unknown vqa status" and msg not in seen
+        seen.add(msg)
+    assert lib.vqa_strerror(-99) == b"unknown vqa status"
+
+
+def test_decode_host_side_queries(lib):
+    # 512 (b,h) units, 32k keys: splits are chosen so there are thousands of workgroups
+    s = lib.vqa_decode_default_splits(16, 32, 32768)
+    assert 1 <= s <= 32 and s * 512 >= 2048
+    assert lib.vqa_decode_default_splits(1, 1, 10) == 1
+    small = lib.vqa_decode_workspace_bytes(1, 1, 64, 128, 4, 256, 1)
+    big = lib.vqa_decode_workspace_bytes(16, 32, 32768, 128, 4, 256, 8)
+    assert 0 < small < big
+    # LUT (B*H*M*256 fp32) + partial states (B*H*S*(D+2) fp32), each 256-byte aligned
+    assert big >= 512 * 4 * 256 * 4 + 512 * 8 * 130 * 4
+
+
+def test_decode_rejects_bad_arguments_before_any_launch(lib):
+    strides = _lib.strides_array(*([0] * 12))
+    args = dict(B=1, H=1, N=8, D=128, M=4, K=256)
+
+    def call(q=1, codes=1, cb=1, v=1, out=1, ws=256, ws_bytes=1 << 20, **kw):
+        a = dict(args, **kw)
+        return lib.vqa_decode_bf16(q, codes, cb, v, out, None, ws, ws_bytes, a["B"], a["H"], a["N"], a["D"], a["M"],
+                                   a["K"], strides, 1.0, 1, None)
+
+    assert call(q=None) == -1                      # VQA_ERR_NULL_POINTER
+    assert call(q=16, cb=16, v=16, N=0) == -2      # VQA_ERR_BAD_SHAPE
+    assert call(q=16, cb=16, v=16, D=96) == -3     # VQA_ERR_UNSUPPORTED_HEAD_DIM
+    assert call(q=16, cb=16, v=16, M=3) == -4      # VQA_ERR_UNSUPPORTED_CODEBOOK
+    assert call(q=16, cb=16, v=16, K=257) == -4
+    assert call(q=18, cb=16, v=16) == -5           # VQA_ERR_MISALIGNED
+    assert call(q=16, cb=16, v=16, codes=4, ws_bytes=8) == -6  # VQA_ERR_WORKSPACE_TOO_SMALL
+
+
+def test_ops_refuse_cpu_tensors():
+    import torch
+
+    from vqtree_amd.ops.attn_vq import attn_vq_decode
+
+    q = torch.zeros(1, 1, 1, 128, dtype=torch.bfloat16)
+    with pytest.raises(_lib.VqaError):
+        attn_vq_decode(q, torch.zeros(1, 1, 8, 4, dtype=torch.uint8), torch.zeros(1, 4, 256, 128, dtype=torch.bfloat16),
+                       torch.zeros(1, 1, 8, 128, dtype=torch.bfloat16))

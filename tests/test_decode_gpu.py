@@ -1,0 +1,106 @@
+"""GPU parity of the seqlen_q = 1 VQ-attention kernel against the CPU oracle (through the C ABI via ctypes)."""
+import math
+
+import pytest
+import torch
+
+import oracle
+from tests.util import assert_close_16, assert_close_lse
+from vqtree_amd.ops.attn_vq import attn_vq_decode
+from vqtree_amd.synthetic import decode_case
+
+pytestmark = pytest.mark.gpu
+
+
+def _check(case, num_splits=0, what=""):
+    print(f"decode case {what} q{tuple(case.q.shape)} codes{tuple(case.codes.shape)} splits={num_splits}", flush=True)
+    out, lse = attn_vq_decode(case.q, case.codes, case.codebooks, case.v, softmax_scale=case.softmax_scale,
+                              return_lse=True, num_splits=num_splits)
+    torch.cuda.synchronize()
+    want, want_lse = oracle.attn_vq_decode(case.q, case.codes, case.codebooks, case.v, case.softmax_scale)
+    assert out.dtype == case.q.dtype and out.shape == case.q.shape
+    assert_close_16(out, want, what)
+    assert_close_lse(lse, want_lse)
+
+
+@pytest.mark.parametrize("N", [1, 5, 63, 64, 65, 255, 256, 257, 1000, 4097])
+def test_ragged_lengths(N):
+    _check(decode_case(2, 3, N, 128, 4, seed=N), what=f"N={N}")
+
+
+@pytest.mark.parametrize("splits", [1, 2, 3, 7, 16])
+def test_split_counts(splits):
+    # more splits than 256-key chunks leaves some splits empty: they must merge as no-ops
+    _check(decode_case(1, 4, 1500, 128, 4, seed=7), num_splits=splits, what=f"splits={splits}")
+
+
+@pytest.mark.parametrize("D,M,K", [(128, 1, 256), (128, 2, 256), (128, 8, 256), (64, 4, 256), (64, 1, 100), (128, 4, 37),
+                                   (64, 8, 256), (64, 2, 16)])
+def test_codebook_shapes(D, M, K):
+    _check(decode_case(2, 2, 777, D, M, K, seed=D + M + K), what=f"D={D} M={M} K={K}")
+
+
+def test_f16():
+    _check(decode_case(2, 2, 900, 128, 4, dtype=torch.float16, seed=11), what="f16")
+    _check(decode_case(1, 2, 300, 64, 2, dtype=torch.float16, seed=12), what="f16 D64")
+
+
+def test_batch_larger_than_one_lut_tile():
+    # the lookup-table kernel sweeps the batch 16 rows at a time
+    _check(decode_case(19, 2, 130, 128, 4, seed=13), what="B=19")
+
+
+def test_strided_v_and_q():
+    # V given as a [B,N,H,D] buffer viewed as [B,H,N,D] (row stride H*D), q as a slice of a longer sequence
+    case = decode_case(2, 4, 600, 128, 4, seed=14)
+    v_bnhd = case.v.transpose(1, 2).contiguous()
+    q_long = torch.randn(2, 4, 5, 128, device="cuda").to(torch.bfloat16)
+    q_long[:, :, 3:4] = case.q
+    case.v = v_bnhd.transpose(1, 2)
+    case.q = q_long[:, :, 3:4]
+    assert not case.v.is_contiguous() and not case.q.is_contiguous()
+    _check(case, what="strided")
+
+
+def test_zero_codebooks_give_mean_of_v():
+    # every score is 0: the kernel reduces to a streaming mean of V, a closed form independent of the oracle
+    case = decode_case(2, 2, 3000, 128, 4, seed=15)
+    case.codebooks.zero_()
+    out, lse = attn_vq_decode(case.q, case.codes, case.codebooks, case.v, return_lse=True)
+    want = case.v.float().mean(dim=2, keepdim=True)
+    assert torch.allclose(out.float(), want, atol=4e-3)
+    assert torch.allclose(lse, torch.full_like(lse, math.log2(3000)), atol=1e-4)
+
+
+def test_dominant_key_selects_its_value_row():
+    case = decode_case(1, 2, 2048, 128, 1, seed=16)
+    case.codebooks.zero_()
+    case.codebooks[:, 0, 9] = (case.q[0, :, 0] * 4).to(case.codebooks.dtype)  # aligned with q, huge score
+    case.codes.zero_()
+    case.codes[0, 0, 1234, 0] = 9
+    case.codes[0, 1, 77, 0] = 9
+    out = attn_vq_decode(case.q, case.codes, case.codebooks, case.v)
+    assert torch.equal(out[0, 0, 0], case.v[0, 0, 1234]) and torch.equal(out[0, 1, 0], case.v[0, 1, 77])
+
+
+def test_large_scores_do_not_overflow():
+    case = decode_case(1, 2, 1024, 128, 4, seed=17, cb_std=3.0)
+    _check(case, what="large scores")
+
+
+def test_full_size_sampled_units():
+    """Benchmark shape (B16 H32 N32768 D128 M4): every output finite, sampled (b,h) units checked against the
+    oracle, and the split count does not change the result beyond rounding."""
+    from vqtree_amd.synthetic import decode_c2
+
+    case = decode_c2()
+    out, lse = attn_vq_decode(case.q, case.codes, case.codebooks, case.v, return_lse=True)
+    out2 = attn_vq_decode(case.q, case.codes, case.codebooks, case.v, num_splits=3)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out.float()).all() and torch.isfinite(lse).all()
+    assert (out.float() - out2.float()).abs().max() <= 2e-3
+    for b, h in [(0, 0), (3, 17), (15, 31), (8, 5)]:
+        want, want_lse = oracle.attn_vq_decode(case.q[b:b + 1, h:h + 1], case.codes[b:b + 1, h:h + 1],
+                                               case.codebooks[h:h + 1], case.v[b:b + 1, h:h + 1], case.softmax_scale)
+        assert_close_16(out[b:b + 1, h:h + 1], want, f"unit {b},{h}")
+        assert_close_lse(lse[b:b + 1, h:h + 1], want_lse)

@@ -1,0 +1,109 @@
+// Internal helpers shared by the gfx950 kernels of libvqattn (not part of the C ABI).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <type_traits>
+
+#define VQA_NO_HIP_STREAM_TYPEDEF
+typedef hipStream_t vqa_stream_t;
+#include "../../include/vqattn.h"
+
+namespace vqa {
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr int kWave = 64;
+
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+
+struct bf16_tag {};
+struct f16_tag {};
+
+// Element-type traits: 16-bit storage, fp32 arithmetic.
+template <typename Tag>
+struct Elem;
+
+template <>
+struct Elem<bf16_tag> {
+    typedef bf16x8_t vec8;
+    // round-to-nearest-even fp32 -> bf16, returned as an fp32 whose low 16 bits are zero
+    static __device__ __forceinline__ float round_keep_f32(float x) {
+        uint32_t u = __builtin_bit_cast(uint32_t, x);
+        u += 0x7fffu + ((u >> 16) & 1u);
+        return __builtin_bit_cast(float, u & 0xffff0000u);
+    }
+    static __device__ __forceinline__ uint16_t to_bits(float x) {
+        return (uint16_t)(__builtin_bit_cast(uint32_t, round_keep_f32(x)) >> 16);
+    }
+    // bits of a value round_keep_f32 already produced
+    static __device__ __forceinline__ uint32_t rounded_to_bits(float x) {
+        return __builtin_bit_cast(uint32_t, x) >> 16;
+    }
+    static __device__ __forceinline__ float from_bits(uint16_t b) {
+        return __builtin_bit_cast(float, (uint32_t)b << 16);
+    }
+    // acc + a.lo*b.lo + a.hi*b.hi with a, b packed pairs
+    static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float acc) {
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, b), acc,
+                                               false);
+    }
+    static __device__ __forceinline__ f32x4_t mfma16(vec8 a, vec8 b, f32x4_t c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ f32x16_t mfma32(vec8 a, vec8 b, f32x16_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+};
+
+template <>
+struct Elem<f16_tag> {
+    typedef f16x8_t vec8;
+    static __device__ __forceinline__ float round_keep_f32(float x) { return (float)(_Float16)x; }
+    static __device__ __forceinline__ uint16_t to_bits(float x) {
+        return __builtin_bit_cast(uint16_t, (_Float16)x);
+    }
+    static __device__ __forceinline__ uint32_t rounded_to_bits(float x) { return to_bits(x); }
+    static __device__ __forceinline__ float from_bits(uint16_t b) { return (float)__builtin_bit_cast(_Float16, b); }
+    static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float acc) {
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, a), __builtin_bit_cast(f16x2_t, b), acc, false);
+    }
+    static __device__ __forceinline__ f32x4_t mfma16(vec8 a, vec8 b, f32x4_t c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ f32x16_t mfma32(vec8 a, vec8 b, f32x16_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+};
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+
+__device__ __forceinline__ float wave_max(float x) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) x = fmaxf(x, __shfl_xor(x, o, 64));
+    return x;
+}
+__device__ __forceinline__ float wave_sum(float x) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) x += __shfl_xor(x, o, 64);
+    return x;
+}
+
+// Orders this wave's LDS writes before its later LDS reads by other lanes (no cross-wave effect).
+__device__ __forceinline__ void wave_lds_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
+}
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+inline int launch_status() { return hipGetLastError() == hipSuccess ? VQA_OK : VQA_ERR_LAUNCH_FAILED; }
+
+}  // namespace vqa

@@ -1,0 +1,431 @@
+// seqlen_q = 1 attention over additive-quantiser key codes (gfx950).
+//
+// Three launches per call, all on the caller's stream:
+//   1. lut_kernel    LUT[b,h,m,c] = sm_scale*log2(e) * <q[b,h], codebooks[h,m,c]>        (MFMA 16x16x32, tiny)
+//   2. main_kernel   one workgroup per (KV split, b*H+h): streams packed uint8 codes and V rows from HBM,
+//                    score_j = sum_m LUT[m][code_jm] from LDS, online base-2 softmax, fp32 accumulation of p*V;
+//                    writes one unnormalised partial state (o[D], m, l) per split
+//   3. merge_kernel  log-sum-exp merge of the split states, normalise, cast, optional lse
+// The main kernel is HBM-bound: per key it reads M code bytes and one D-element V row and nothing else.
+#include "vqa_common.h"
+
+namespace vqa {
+namespace decode {
+
+constexpr int kLutStride = 256;   // LUT entries reserved per codebook (uint8 codes)
+constexpr int kThreads = 256;     // main kernel workgroup: 4 waves
+constexpr int kWaves = kThreads / kWave;
+constexpr int kBatch = 64;        // keys scored per wave per step (one per lane)
+
+struct Strides {
+    int64_t q_b, q_h;
+    int64_t c_b, c_h;
+    int64_t cb_h, cb_m, cb_k;
+    int64_t v_b, v_h, v_n;
+    int64_t o_b, o_h;
+};
+
+// ---------------------------------------------------------------------------------------------------------------
+// 1. lookup table.  One wave owns 16 codewords of one (h, m) and sweeps the batch 16 rows at a time:
+//    C[code, b] = sum_d cb[code, d] * q[b, d] as D/32 MFMA 16x16x32 steps; A and B fragments come straight from
+//    global memory (each lane: 8 contiguous elements of its row).
+// ---------------------------------------------------------------------------------------------------------------
+template <typename Tag, int D>
+__global__ __launch_bounds__(kThreads) void lut_kernel(const uint16_t* __restrict__ q,
+                                                       const uint16_t* __restrict__ cb, float* __restrict__ lut,
+                                                       int B, int H, int M, int K, Strides st, float scale_log2e) {
+    typedef typename Elem<Tag>::vec8 vec8;
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int tile = blockIdx.x * kWaves + wave;  // 16-codeword tile inside this codebook
+    if (tile * 16 >= K) return;
+    const int hm = blockIdx.y;
+    const int h = hm / M, m = hm % M;
+    const int r = lane & 15;   // A row (codeword) / B column (batch row)
+    const int kq = lane >> 4;  // which 8-element slice of each 32-wide k step
+    const int code = min(tile * 16 + r, K - 1);
+    const uint16_t* a_row = cb + h * st.cb_h + m * st.cb_m + (int64_t)code * st.cb_k + kq * 8;
+    vec8 a[D / 32];
+#pragma unroll
+    for (int kk = 0; kk < D / 32; ++kk) a[kk] = *reinterpret_cast<const vec8*>(a_row + kk * 32);
+
+    for (int b0 = 0; b0 < B; b0 += 16) {
+        const int bb = b0 + r;
+        f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+        const uint16_t* b_row = q + (int64_t)min(bb, B - 1) * st.q_b + h * st.q_h + kq * 8;
+#pragma unroll
+        for (int kk = 0; kk < D / 32; ++kk) {
+            vec8 bv = *reinterpret_cast<const vec8*>(b_row + kk * 32);
+            acc = Elem<Tag>::mfma16(a[kk], bv, acc);
+        }
+        // acc[i]: codeword row 4*kq + i, batch column r
+        if (bb < B) {
+            float* dst = lut + ((int64_t)(bb * H + h) * M + m) * kLutStride + tile * 16 + kq * 4;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (tile * 16 + kq * 4 + i < K) dst[i] = acc[i] * scale_log2e;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// 2. main streaming kernel
+// ---------------------------------------------------------------------------------------------------------------
+template <int M>
+struct CodeWord;
+template <>
+struct CodeWord<1> {
+    typedef uint8_t type;
+};
+template <>
+struct CodeWord<2> {
+    typedef uint16_t type;
+};
+template <>
+struct CodeWord<4> {
+    typedef uint32_t type;
+};
+template <>
+struct CodeWord<8> {
+    typedef uint2 type;
+};
+
+template <int M>
+__device__ __forceinline__ float score_from_lut(const float* s_lut, typename CodeWord<M>::type cw) {
+    if constexpr (M == 8) {
+        float s = 0.f;
+#pragma unroll
+        for (int m = 0; m < 4; ++m) s += s_lut[m * kLutStride + ((cw.x >> (8 * m)) & 0xffu)];
+#pragma unroll
+        for (int m = 0; m < 4; ++m) s += s_lut[(4 + m) * kLutStride + ((cw.y >> (8 * m)) & 0xffu)];
+        return s;
+    } else {
+        const uint32_t w = cw;
+        float s = 0.f;
+#pragma unroll
+        for (int m = 0; m < M; ++m) s += s_lut[m * kLutStride + ((w >> (8 * m)) & 0xffu)];
+        return s;
+    }
+}
+
+// Lane layout inside a wave: LPR = D/8 lanes cover one V row with 16-byte loads, so one load instruction covers
+// G = 64/LPR consecutive rows; a 64-key batch takes R = 64/G loads per lane.  Lane (g, c) accumulates rows
+// {i*G + g} into its 8 output elements c*8..c*8+7; the G row groups are summed once at the end.
+//
+// Each wave walks batches k0, k0 + 256, ... of its split.  The R row buffers roll: as soon as row i of the current
+// batch has been accumulated its registers receive row i of the next batch, so every wave keeps R 16-byte loads per
+// lane in flight at all times with only R*4 buffer registers.  A ragged last batch is moved back to end exactly at
+// the split end (keys already consumed get weight zero), so no load in the loop needs clamping.
+template <typename Tag, int D, int M>
+__global__ __launch_bounds__(kThreads, 3) void main_kernel(const uint8_t* __restrict__ codes,
+                                                           const uint16_t* __restrict__ v,
+                                                           const float* __restrict__ lut,
+                                                           float* __restrict__ part_o, float* __restrict__ part_ml,
+                                                           int H, int N, int S, int keys_per_split, Strides st) {
+    constexpr int LPR = D / 8;
+    constexpr int G = kWave / LPR;
+    constexpr int R = kBatch / G;
+    constexpr int kStep = kWaves * kBatch;
+    typedef typename CodeWord<M>::type code_t;
+
+    __shared__ float s_lut[M * kLutStride];
+    __shared__ __attribute__((aligned(16))) float s_p[kWaves][kBatch];
+    __shared__ float s_red[kWaves][G][D];
+    __shared__ float s_m[kWaves];
+    __shared__ float s_l[kWaves];
+
+    const int split = blockIdx.x;
+    const int bh = blockIdx.y;
+    const int b = bh / H, h = bh % H;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int g = lane / LPR, c = lane % LPR;
+
+    for (int i = tid; i < M * kLutStride; i += kThreads) s_lut[i] = lut[(int64_t)bh * M * kLutStride + i];
+    __syncthreads();
+
+    const int k_begin = split * keys_per_split;
+    const int k_end = min(N, k_begin + keys_per_split);
+    const code_t* code_base = reinterpret_cast<const code_t*>(codes + b * st.c_b + h * st.c_h);
+    const char* v_bh = reinterpret_cast<const char*>(v + b * st.v_b + h * st.v_h);
+    const int64_t row_bytes = st.v_n * 2;
+    const uint32_t lane_off = (uint32_t)(g * row_bytes) + c * 16;  // this lane's slice of row g of a batch
+    const uint32_t grp_bytes = (uint32_t)(G * row_bytes);          // distance between consecutive loads
+
+    float m_run = -INFINITY;
+    float l_run = 0.f;
+    float acc[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+
+    uint4 buf[R];
+    code_t cw_cur, cw_nxt;
+
+    const int k0 = k_begin + wave * kBatch;
+    const int n_batches = k0 < k_end ? (k_end - k0 + kStep - 1) / kStep : 0;
+    // batch j scores keys [valid_from, k_end) of the 64 loaded from load_from
+    auto batch_bounds = [&](int j, int& load_from, int& valid_from) {
+        valid_from = k0 + j * kStep;
+        load_from = (valid_from + kBatch <= k_end) ? valid_from : max(k_end - kBatch, 0);
+    };
+    auto load_code = [&](int load_from) { return code_base[min(load_from + lane, N - 1)]; };
+
+    auto process = [&](auto prefetch, int load_from, int valid_from, int next_load_from) {
+        constexpr bool kPrefetch = decltype(prefetch)::value;
+        float s = score_from_lut<M>(s_lut, cw_cur);
+        const int key = load_from + lane;
+        s = (key >= valid_from && key < k_end) ? s : -INFINITY;
+        if constexpr (kPrefetch) cw_nxt = load_code(next_load_from);
+        const float m_new = fmaxf(m_run, wave_max(s));
+        if (m_new > m_run) {  // same outcome in every lane of the wave
+            const float alpha = fast_exp2(m_run - m_new);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[e] *= alpha;
+            l_run *= alpha;
+            m_run = m_new;
+        }
+        float p = (s == -INFINITY) ? 0.f : fast_exp2(s - m_run);
+        p = Elem<Tag>::round_keep_f32(p);  // P is rounded to the V type before P.V; l sums the same values
+        l_run += p;
+        // key lane -> slot (key % G) * R + key / G, so row group g finds its R weights contiguous
+        s_p[wave][(lane % G) * R + lane / G] = p;
+        wave_lds_sync();
+        float pr[R];
+#pragma unroll
+        for (int i = 0; i < R; i += 4) {
+            const f32x4_t t = *reinterpret_cast<const f32x4_t*>(&s_p[wave][g * R + i]);
+            pr[i] = t[0];
+            pr[i + 1] = t[1];
+            pr[i + 2] = t[2];
+            pr[i + 3] = t[3];
+        }
+        wave_lds_sync();
+        const char* next_base = v_bh + (int64_t)next_load_from * row_bytes;
+#pragma unroll
+        for (int i = 0; i < R; ++i) {
+            // packed weight pairs (p, 0) and (0, p) in the V element type
+            const uint32_t pbits = Elem<Tag>::rounded_to_bits(pr[i]);
+            const uint32_t p_lo = pbits, p_hi = pbits << 16;
+            const uint32_t w[4] = {buf[i].x, buf[i].y, buf[i].z, buf[i].w};
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                acc[2 * d] = Elem<Tag>::dot2(w[d], p_lo, acc[2 * d]);
+                acc[2 * d + 1] = Elem<Tag>::dot2(w[d], p_hi, acc[2 * d + 1]);
+            }
+            if constexpr (kPrefetch) {
+                buf[i] = *reinterpret_cast<const uint4*>(next_base + (lane_off + i * grp_bytes));
+                __builtin_amdgcn_sched_barrier(0);  // keep the reload right behind the row it replaces
+            }
+        }
+        if constexpr (kPrefetch) cw_cur = cw_nxt;
+    };
+
+    if (n_batches > 0) {
+        int load_from, valid_from;
+        batch_bounds(0, load_from, valid_from);
+        cw_cur = load_code(load_from);
+        const char* base = v_bh + (int64_t)load_from * row_bytes;
+        if (N >= kBatch) {
+#pragma unroll
+            for (int i = 0; i < R; ++i)
+                buf[i] = *reinterpret_cast<const uint4*>(base + (lane_off + i * grp_bytes));
+        } else {  // fewer keys than one batch in the whole sequence: clamp rows (their weight is zero)
+#pragma unroll
+            for (int i = 0; i < R; ++i)
+                buf[i] = *reinterpret_cast<const uint4*>(v_bh + (int64_t)min(i * G + g, N - 1) * row_bytes + c * 16);
+        }
+        for (int j = 0; j + 1 < n_batches; ++j) {
+            int next_load_from, next_valid_from;
+            batch_bounds(j + 1, next_load_from, next_valid_from);
+            process(std::true_type{}, load_from, valid_from, next_load_from);
+            load_from = next_load_from;
+            valid_from = next_valid_from;
+        }
+        process(std::false_type{}, load_from, valid_from, load_from);
+    }
+
+    // combine the G row groups of each wave and the waves of the workgroup
+    const float l_wave = wave_sum(l_run);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) s_red[wave][g][c * 8 + e] = acc[e];
+    if (lane == 0) {
+        s_m[wave] = m_run;
+        s_l[wave] = l_wave;
+    }
+    __syncthreads();
+    if (tid < D) {
+        float m_all = s_m[0];
+#pragma unroll
+        for (int w = 1; w < kWaves; ++w) m_all = fmaxf(m_all, s_m[w]);
+        float o = 0.f, l = 0.f;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) {
+            const float wgt = (s_m[w] == -INFINITY) ? 0.f : fast_exp2(s_m[w] - m_all);
+            float t = 0.f;
+#pragma unroll
+            for (int gg = 0; gg < G; ++gg) t += s_red[w][gg][tid];
+            o += wgt * t;
+            l += wgt * s_l[w];
+        }
+        const int64_t slot = (int64_t)bh * S + split;
+        part_o[slot * D + tid] = o;
+        if (tid == 0) {
+            part_ml[slot * 2] = m_all;
+            part_ml[slot * 2 + 1] = l;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// 3. merge of the split states
+// ---------------------------------------------------------------------------------------------------------------
+template <typename Tag, int D>
+__global__ __launch_bounds__(D) void merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                                  uint16_t* __restrict__ out, float* __restrict__ lse, int H, int S,
+                                                  Strides st) {
+    const int bh = blockIdx.x;
+    const int b = bh / H, h = bh % H;
+    const int d = threadIdx.x;
+    float m_all = -INFINITY;
+    for (int s = 0; s < S; ++s) m_all = fmaxf(m_all, part_ml[((int64_t)bh * S + s) * 2]);
+    float o = 0.f, l = 0.f;
+    for (int s = 0; s < S; ++s) {
+        const int64_t slot = (int64_t)bh * S + s;
+        const float ms = part_ml[slot * 2];
+        const float wgt = (ms == -INFINITY) ? 0.f : fast_exp2(ms - m_all);
+        o += wgt * part_o[slot * D + d];
+        l += wgt * part_ml[slot * 2 + 1];
+    }
+    const float res = l > 0.f ? o / l : 0.f;
+    out[b * st.o_b + h * st.o_h + d] = Elem<Tag>::to_bits(res);
+    if (lse != nullptr && d == 0) lse[bh] = l > 0.f ? m_all + fast_log2(l) : -INFINITY;
+}
+
+inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+struct Workspace {
+    size_t lut_off, po_off, pml_off, total;
+};
+
+inline Workspace plan(int B, int H, int D, int M, int S) {
+    Workspace w;
+    const size_t bh = (size_t)B * H;
+    w.lut_off = 0;
+    w.po_off = align_up(bh * M * kLutStride * sizeof(float), 256);
+    w.pml_off = w.po_off + align_up(bh * S * D * sizeof(float), 256);
+    w.total = w.pml_off + align_up(bh * S * 2 * sizeof(float), 256);
+    return w;
+}
+
+inline int default_splits(int B, int H, int N) {
+    // aim for ~16 workgroups per CU (256 CUs) so the tail is short, but keep >= 1024 keys per split
+    const int64_t bh = (int64_t)B * H;
+    if (bh <= 0 || N <= 0) return 1;
+    int64_t s = (4096 + bh - 1) / bh;
+    const int64_t max_s = (N + 1023) / 1024;
+    if (s > max_s) s = max_s;
+    if (s < 1) s = 1;
+    if (s > 256) s = 256;
+    return (int)s;
+}
+
+template <typename Tag, int D, int M>
+int launch_main(const uint8_t* codes, const uint16_t* v, const float* lut, float* po, float* pml, int B, int H, int N,
+                int S, int kps, const Strides& st, hipStream_t stream) {
+    hipLaunchKernelGGL((main_kernel<Tag, D, M>), dim3(S, B * H), dim3(kThreads), 0, stream, codes, v, lut, po, pml, H,
+                       N, S, kps, st);
+    return launch_status();
+}
+
+template <typename Tag, int D>
+int run_d(const void* q, const uint8_t* codes, const void* codebooks, const void* v, void* out, float* lse,
+          void* workspace, int B, int H, int N, int M, int K, const Strides& st, float sm_scale, int S,
+          hipStream_t stream) {
+    const Workspace ws = plan(B, H, D, M, S);
+    char* base = static_cast<char*>(workspace);
+    float* lut = reinterpret_cast<float*>(base + ws.lut_off);
+    float* po = reinterpret_cast<float*>(base + ws.po_off);
+    float* pml = reinterpret_cast<float*>(base + ws.pml_off);
+    const uint16_t* q16 = static_cast<const uint16_t*>(q);
+    const uint16_t* cb16 = static_cast<const uint16_t*>(codebooks);
+    const uint16_t* v16 = static_cast<const uint16_t*>(v);
+
+    const int tiles = (K + 15) / 16;
+    hipLaunchKernelGGL((lut_kernel<Tag, D>), dim3((tiles + kWaves - 1) / kWaves, H * M), dim3(kThreads), 0, stream,
+                       q16, cb16, lut, B, H, M, K, st, sm_scale * kLog2e);
+    int rc = launch_status();
+    if (rc != VQA_OK) return rc;
+
+    // keys per split: a multiple of the workgroup's 256-key stride so only the last split is ragged
+    int kps = (N + S - 1) / S;
+    kps = (kps + kThreads - 1) / kThreads * kThreads;
+    switch (M) {
+        case 1: rc = launch_main<Tag, D, 1>(codes, v16, lut, po, pml, B, H, N, S, kps, st, stream); break;
+        case 2: rc = launch_main<Tag, D, 2>(codes, v16, lut, po, pml, B, H, N, S, kps, st, stream); break;
+        case 4: rc = launch_main<Tag, D, 4>(codes, v16, lut, po, pml, B, H, N, S, kps, st, stream); break;
+        case 8: rc = launch_main<Tag, D, 8>(codes, v16, lut, po, pml, B, H, N, S, kps, st, stream); break;
+        default: return VQA_ERR_UNSUPPORTED_CODEBOOK;
+    }
+    if (rc != VQA_OK) return rc;
+    hipLaunchKernelGGL((merge_kernel<Tag, D>), dim3(B * H), dim3(D), 0, stream, po, pml,
+                       static_cast<uint16_t*>(out), lse, H, S, st);
+    return launch_status();
+}
+
+template <typename Tag>
+int run(const void* q, const uint8_t* codes, const void* codebooks, const void* v, void* out, float* lse,
+        void* workspace, size_t workspace_bytes, int B, int H, int N, int D, int M, int K, const int64_t* strides,
+        float sm_scale, int num_splits, hipStream_t stream) {
+    if (!q || !codes || !codebooks || !v || !out || !workspace || !strides) return VQA_ERR_NULL_POINTER;
+    if (B <= 0 || H <= 0 || N <= 0) return VQA_ERR_BAD_SHAPE;
+    if (D != 64 && D != 128) return VQA_ERR_UNSUPPORTED_HEAD_DIM;
+    if ((M != 1 && M != 2 && M != 4 && M != 8) || K < 1 || K > 256) return VQA_ERR_UNSUPPORTED_CODEBOOK;
+    Strides st;
+    st.q_b = strides[0], st.q_h = strides[1];
+    st.c_b = strides[2], st.c_h = strides[3];
+    st.cb_h = strides[4], st.cb_m = strides[5], st.cb_k = strides[6];
+    st.v_b = strides[7], st.v_h = strides[8], st.v_n = strides[9];
+    st.o_b = strides[10], st.o_h = strides[11];
+    // 16-byte vector loads of q / codebook / V rows; M-byte loads of packed code rows
+    if (!aligned16(q) || !aligned16(codebooks) || !aligned16(v) || ((uintptr_t)workspace & 255u))
+        return VQA_ERR_MISALIGNED;
+    if ((st.q_b | st.q_h | st.cb_h | st.cb_m | st.cb_k | st.v_b | st.v_h | st.v_n) & 7) return VQA_ERR_MISALIGNED;
+    if (((uintptr_t)codes | (uintptr_t)st.c_b | (uintptr_t)st.c_h) & (uintptr_t)(M - 1)) return VQA_ERR_MISALIGNED;
+    int S = num_splits > 0 ? num_splits : default_splits(B, H, N);
+    if (S > 65535 || (int64_t)B * H > 65535) return VQA_ERR_BAD_ARGUMENT;
+    if (workspace_bytes < plan(B, H, D, M, S).total) return VQA_ERR_WORKSPACE_TOO_SMALL;
+    if (D == 64)
+        return run_d<Tag, 64>(q, codes, codebooks, v, out, lse, workspace, B, H, N, M, K, st, sm_scale, S, stream);
+    return run_d<Tag, 128>(q, codes, codebooks, v, out, lse, workspace, B, H, N, M, K, st, sm_scale, S, stream);
+}
+
+}  // namespace decode
+}  // namespace vqa
+
+extern "C" {
+
+int vqa_decode_default_splits(int B, int H, int N) { return vqa::decode::default_splits(B, H, N); }
+
+size_t vqa_decode_workspace_bytes(int B, int H, int N, int D, int M, int K, int num_splits) {
+    (void)K;
+    if (B <= 0 || H <= 0 || N <= 0 || D <= 0 || M <= 0) return 0;
+    const int S = num_splits > 0 ? num_splits : vqa::decode::default_splits(B, H, N);
+    return vqa::decode::plan(B, H, D, M, S).total;
+}
+
+int vqa_decode_bf16(const void* q, const uint8_t* codes, const void* codebooks, const void* v, void* out, float* lse,
+                    void* workspace, size_t workspace_bytes, int B, int H, int N, int D, int M, int K,
+                    const int64_t* strides, float sm_scale, int num_splits, vqa_stream_t stream) {
+    return vqa::decode::run<vqa::bf16_tag>(q, codes, codebooks, v, out, lse, workspace, workspace_bytes, B, H, N, D, M,
+                                           K, strides, sm_scale, num_splits, stream);
+}
+
+int vqa_decode_f16(const void* q, const uint8_t* codes, const void* codebooks, const void* v, void* out, float* lse,
+                   void* workspace, size_t workspace_bytes, int B, int H, int N, int D, int M, int K,
+                   const int64_t* strides, float sm_scale, int num_splits, vqa_stream_t stream) {
+    return vqa::decode::run<vqa::f16_tag>(q, codes, codebooks, v, out, lse, workspace, workspace_bytes, B, H, N, D, M,
+                                          K, strides, sm_scale, num_splits, stream);
+}
+
+}  // extern "C"
