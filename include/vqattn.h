@@ -76,6 +76,114 @@ int vqa_decode_f16(const void* q, const uint8_t* codes, const void* codebooks, c
                    void* workspace, size_t workspace_bytes, int B, int H, int N, int D, int M, int K,
                    const int64_t* strides, float sm_scale, int num_splits, vqa_stream_t stream);
 
+/* ------------------------------------------------------------------------------------------------------------------
+ * Sliding-window exact attention, seqlen_q == seqlen_k == N, causal.  One kernel, three masks:
+ *
+ *   mode 0 (VQA_LOCAL_STRICT)  key j visible iff j <= i and i - j <= window
+ *                              replaces ops/triton_fused_local_attn.py:254-262 (flash_attn_func)
+ *   mode 1 (VQA_LOCAL_LOOSE)   key j visible iff j <= i and j >= floor(i/128)*128 - window  (whole 128-blocks)
+ *                              replaces ops/triton_fused_local_attn2.py:249-256
+ *   mode 2 (VQA_LOCAL_REROPE)  visible as mode 1; score = q1.k1 when i - j <= window, else q2.k2
+ *                              replaces ops/triton_fused_local_attn_rerope.py:287-294
+ *
+ *   q1,q2,k1,k2,v,out: [B,H,N,D]-addressable bf16/f16 tensors; strides[0..17] = (b,h,n) element strides of
+ *   q1, q2, k1, k2, v, out in this order (a [B,N,H,D] tensor is passed with its h and n strides swapped).
+ *   q2/k2 are read only in mode 2 (may be NULL otherwise).  Inputs 16-byte aligned rows, out 8-byte aligned rows.
+ *   lse: [B,H,N] contiguous float, base 2, nullable.
+ * ------------------------------------------------------------------------------------------------------------------ */
+#define VQA_LOCAL_STRICT 0
+#define VQA_LOCAL_LOOSE 1
+#define VQA_LOCAL_REROPE 2
+#define VQA_LOCAL_NUM_STRIDES 18
+
+int vqa_local_attn_bf16(const void* q1, const void* q2, const void* k1, const void* k2, const void* v, void* out,
+                        float* lse, int B, int H, int N, int D, const int64_t* strides, int window, int mode,
+                        float sm_scale, vqa_stream_t stream);
+
+int vqa_local_attn_f16(const void* q1, const void* q2, const void* k1, const void* k2, const void* v, void* out,
+                       float* lse, int B, int H, int N, int D, const int64_t* strides, int window, int mode,
+                       float sm_scale, vqa_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------------------------------
+ * Full-context ReRoPE attention: score(i,j) = q1_i.k1_j if |i - j| < window (strict) else q2_i.k2_j; keys j <= i
+ * when `causal`, all keys otherwise.  Replaces ops/triton_fused_attn_rerope.py:185-233 (attention).
+ * Arguments as vqa_local_attn_* (same 18 strides).
+ * ------------------------------------------------------------------------------------------------------------------ */
+int vqa_rerope_full_bf16(const void* q1, const void* q2, const void* k1, const void* k2, const void* v, void* out,
+                         float* lse, int B, int H, int N, int D, const int64_t* strides, int window, int causal,
+                         float sm_scale, vqa_stream_t stream);
+
+int vqa_rerope_full_f16(const void* q1, const void* q2, const void* k1, const void* k2, const void* v, void* out,
+                        float* lse, int B, int H, int N, int D, const int64_t* strides, int window, int causal,
+                        float sm_scale, vqa_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------------------------------
+ * Prefill attention over additive-quantiser key codes with an optional exact sliding window (seqlen_q == seqlen_k).
+ * Generalises what vq_attn_forward computes (ops/triton_fused_vq_attn.py:190-251, naive form ops/attn_vq.py:308-333)
+ * from one codebook to M, in one fused pass (no separate merge):
+ *
+ *   keys j <  boundary(i)          quantised:  score = qf_i . sum_m codebooks[h,m,codes[b,h,j,m]],  qf = q2 if given else q
+ *   keys boundary(i) <= j < i - W  exact strip: score = q2_i . k2_j when q2 and k2 are given, else q_i . k_exact_j
+ *   keys i - W <= j <= i           exact window: score = q_i . k_exact_j
+ *   boundary(i) = max(0, floor((i - W)/128)*128)  (boundary_mode 0, the reference's block rule)
+ *               = max(0, i - W)                   (boundary_mode 1)
+ *   k_exact == NULL: every visible key is quantised (window ignored); causal == 0 requires k_exact == NULL.
+ *
+ *   strides[0..22]: q(b,h,n) codes(b,h) codebooks(h,m,k) v(b,h,n) k_exact(b,h,n) q2(b,h,n) k2(b,h,n) out(b,h,n);
+ *   code rows are packed (stride(n) = M).  M in [1,16], K <= 256, D in {64,128}.
+ *   workspace: >= vqa_prefill_workspace_bytes(B,H,N,D) bytes, 256-byte aligned (holds the reconstructed keys).
+ * ------------------------------------------------------------------------------------------------------------------ */
+#define VQA_BOUNDARY_BLOCK 0
+#define VQA_BOUNDARY_EXACT 1
+#define VQA_PREFILL_NUM_STRIDES 23
+
+size_t vqa_prefill_workspace_bytes(int B, int H, int N, int D);
+
+int vqa_prefill_bf16(const void* q, const uint8_t* codes, const void* codebooks, const void* v, const void* k_exact,
+                     const void* q2, const void* k2, void* out, float* lse, void* workspace, size_t workspace_bytes,
+                     int B, int H, int N, int D, int M, int K, const int64_t* strides, int window, int boundary_mode,
+                     int causal, float sm_scale, vqa_stream_t stream);
+
+int vqa_prefill_f16(const void* q, const uint8_t* codes, const void* codebooks, const void* v, const void* k_exact,
+                    const void* q2, const void* k2, void* out, float* lse, void* workspace, size_t workspace_bytes,
+                    int B, int H, int N, int D, int M, int K, const int64_t* strides, int window, int boundary_mode,
+                    int causal, float sm_scale, vqa_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------------------------------
+ * Count-weighted far-context kernel of the single-codebook formulation.  Replaces _vq_fwd_kernel
+ * (ops/triton_fused_vq_attn.py:88-187) including the host-side zero / -inf initialisation (:214-215):
+ * rows i < window + 128 get out = 0, lse = -inf; query tile t (rows window+128+128t ..) attends over the C codewords
+ * with cnt[b,h,t,:] and the per-code V prefix sums v_vq[b,h,vi[b,h,t,c],:].
+ *
+ *   strides[0..16]: q2(b,h,n) k_vq(h,c) k_vq_cnt(b,h,t) v_vq(b,h,n) vi(b,h,t) out(b,h,n); k_vq_cnt has q2's element
+ *   type, vi is int64; both have unit stride along c.  lse: [B,H,N] contiguous float, base 2, nullable.
+ * ------------------------------------------------------------------------------------------------------------------ */
+#define VQA_VQCOUNT_NUM_STRIDES 17
+
+int vqa_vqcount_fwd_bf16(const void* q2, const void* k_vq, const void* k_vq_cnt, const void* v_vq, const int64_t* vi,
+                         void* out, float* lse, int B, int H, int N, int D, int C, const int64_t* strides, int window,
+                         float sm_scale, vqa_stream_t stream);
+
+int vqa_vqcount_fwd_f16(const void* q2, const void* k_vq, const void* k_vq_cnt, const void* v_vq, const int64_t* vi,
+                        void* out, float* lse, int B, int H, int N, int D, int C, const int64_t* strides, int window,
+                        float sm_scale, vqa_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------------------------------
+ * In-place merge of two attention states with base-2 log-sum-exp: m = max(s, s'), o <- (o 2^(s-m) + o' 2^(s'-m)) /
+ * (2^(s-m) + 2^(s'-m)), s <- m + log2(2^(s-m) + 2^(s'-m)); a side with s = -inf is ignored.
+ * Replaces flashinfer.merge_state_in_place as called at ops/triton_fused_vq_attn.py:246-250.
+ *
+ *   o, o_other: [B,H,N,D]-addressable; s, s_other: [B,H,N]-addressable float; strides[0..11] = (b,h,n) of
+ *   o, s, o_other, s_other.  (flashinfer's [N, B*H, D] / [N, B*H] layout is B = 1, H = B*H with n outermost.)
+ * ------------------------------------------------------------------------------------------------------------------ */
+#define VQA_MERGE_NUM_STRIDES 12
+
+int vqa_merge_state_inplace_bf16(void* o, float* s, const void* o_other, const float* s_other, int B, int H, int N,
+                                 int D, const int64_t* strides, vqa_stream_t stream);
+
+int vqa_merge_state_inplace_f16(void* o, float* s, const void* o_other, const float* s_other, int B, int H, int N,
+                                int D, const int64_t* strides, vqa_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,237 @@
+"""GPU parity of the sliding-window / ReRoPE / VQ-prefill MFMA kernels against the CPU oracle."""
+import math
+
+import pytest
+import torch
+
+import oracle
+from tests.util import assert_close_16, assert_close_lse
+from vqtree_amd.ops import (triton_fused_attn_rerope, triton_fused_local_attn, triton_fused_local_attn2,
+                            triton_fused_local_attn_rerope, triton_fused_vq_attn)
+from vqtree_amd.ops.attn_vq import attn_vq_prefill
+
+pytestmark = pytest.mark.gpu
+
+
+def _randn(*shape, seed, std=1.0, dtype=torch.bfloat16):
+    g = torch.Generator("cpu").manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * std).to(dtype)
+
+
+def _bnhd(x):  # [B,H,N,D] -> contiguous [B,N,H,D]
+    return x.transpose(1, 2).contiguous()
+
+
+def _say(msg):
+    print(msg, flush=True)
+
+
+# ------------------------------------------------------------------ strict / loose / rerope-local windows
+@pytest.mark.parametrize("N", [2048, 2013])
+@pytest.mark.parametrize("mode", ["strict", "loose", "rerope"])
+def test_reference_selfcheck_shapes(mode, N):
+    """The shapes of the reference's own self-checks: Z=1, H=2, D=64, W=512, sm_scale 0.5, fp16 N(0, 0.5), even and
+    uneven lengths (ops/triton_fused_local_attn.py:265-294, ops/triton_fused_local_attn2.py:277-335)."""
+    _say(f"window selfcheck {mode} N={N}")
+    B, H, D, W, scale = 1, 2, 64, 512, 0.5
+    q, k, v, q2, k2 = (_randn(B, H, N, D, seed=s, std=0.5, dtype=torch.float16) for s in range(5))
+    want, want_lse = oracle.local_attn(q, k, v, W, mode, scale, q2=q2, k2=k2)
+    qd, kd, vd, q2d, k2d = (_bnhd(x).cuda() for x in (q, k, v, q2, k2))
+    if mode == "strict":
+        out, lse = triton_fused_local_attn.flash_attn_func(qd, kd, vd, W, scale), None
+    elif mode == "loose":
+        out, lse = triton_fused_local_attn2.flash_attn_func(qd, kd, vd, W, scale, return_lse=True)
+    else:
+        out, lse = triton_fused_local_attn_rerope.flash_attn_func(qd, q2d, kd, k2d, vd, W, scale, return_lse=True)
+    torch.cuda.synchronize()
+    assert out.shape == (B, N, H, D) and out.is_contiguous()
+    got = out.transpose(1, 2).float().cpu()
+    assert (got - want).abs().max() <= 2e-2  # the reference's acceptance: atol 2e-2, rtol 0
+    assert_close_16(got, want, mode)
+    if lse is not None:
+        assert_close_lse(lse, want_lse)
+
+
+@pytest.mark.parametrize("mode", ["strict", "loose", "rerope"])
+@pytest.mark.parametrize("B,H,N,D,W", [(2, 3, 384, 128, 128), (1, 2, 130, 128, 128), (1, 2, 257, 64, 128),
+                                        (1, 1, 511, 128, 256), (2, 2, 1000, 128, 384), (1, 2, 64, 64, 128),
+                                        (1, 2, 700, 128, 1024), (1, 1, 1, 128, 128)])
+def test_window_modes(mode, B, H, N, D, W):
+    _say(f"window {mode} B{B} H{H} N{N} D{D} W{W}")
+    q, k, v, q2, k2 = (_randn(B, H, N, D, seed=10 + s) for s in range(5))
+    want, want_lse = oracle.local_attn(q, k, v, W, mode, None, q2=q2, k2=k2)
+    qd, kd, vd, q2d, k2d = (_bnhd(x).cuda() for x in (q, k, v, q2, k2))
+    if mode == "strict":
+        out, lse = triton_fused_local_attn.flash_attn_func(qd, kd, vd, W), None
+    elif mode == "loose":
+        out, lse = triton_fused_local_attn2.flash_attn_func(qd, kd, vd, W, return_lse=True)
+    else:
+        out, lse = triton_fused_local_attn_rerope.flash_attn_func(qd, q2d, kd, k2d, vd, W, return_lse=True)
+    torch.cuda.synchronize()
+    assert_close_16(out.transpose(1, 2), want, mode)
+    if lse is not None:
+        assert_close_lse(lse, want_lse)
+
+
+def test_loose_matches_dense_ref_impl_on_device():
+    q, k, v = (_bnhd(_randn(1, 2, 640, 64, seed=20 + s, std=0.5, dtype=torch.float16)).cuda() for s in range(3))
+    out = triton_fused_local_attn2.flash_attn_func(q, k, v, 256, 0.5)
+    ref = triton_fused_local_attn2.local_attn2_ref_impl(q, k, v, 256, 0.5)
+    assert torch.allclose(out.float(), ref.float(), atol=2e-2, rtol=0)
+
+
+def test_window_mask_is_exact():
+    """Bit-exact mask check: V rows are one-hot position markers and all scores are equal, so each output row is
+    (indicator of the visible key set) / (its size) -- any wrongly visible or hidden key changes an element."""
+    N, D, W = 384, 128, 128
+    v = torch.zeros(1, 1, N, D, dtype=torch.bfloat16)
+    v[0, 0, torch.arange(N), torch.arange(N) % D] = 1.0
+    z = torch.zeros(1, 1, N, D, dtype=torch.bfloat16)
+    for mode in ("strict", "loose", "rerope"):
+        vis, _ = oracle.local_visible_mask(N, W, mode)
+        zd, vd = _bnhd(z).cuda(), _bnhd(v).cuda()
+        if mode == "strict":
+            out = triton_fused_local_attn.flash_attn_func(zd, zd, vd, W)
+        elif mode == "loose":
+            out = triton_fused_local_attn2.flash_attn_func(zd, zd, vd, W)
+        else:
+            out = triton_fused_local_attn_rerope.flash_attn_func(zd, zd, zd, zd, vd, W)
+        got = out[0, :, 0].float().cpu()  # [N, D]
+        cnt = vis.sum(1, keepdim=True).float()
+        want = torch.zeros(N, D)
+        for c in range(D):
+            want[:, c] = vis[:, c::D].sum(1)
+        want = want / cnt
+        # one wrongly visible / hidden key moves an element by >= 1/257 = 3.9e-3; 16-bit rounding moves it < 1e-4
+        assert torch.allclose(got, want, atol=3e-4, rtol=0), mode
+
+
+# ------------------------------------------------------------------ full ReRoPE
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("N,D,W", [(2048, 64, 512), (700, 128, 128), (300, 128, 512), (130, 64, 64)])
+def test_rerope_full(causal, N, D, W):
+    """Includes the reference self-check shape Z=1,H=16->2,N=2048,D=64,W=512 fp16 sm_scale 0.5
+    (ops/triton_fused_attn_rerope.py:253-268; it checks the non-causal call)."""
+    _say(f"rerope_full causal={causal} N{N} D{D} W{W}")
+    B, H = 1, 2
+    q1, q2, k1, k2, v = (_randn(B, H, N, D, seed=30 + s, std=0.5, dtype=torch.float16) for s in range(5))
+    want, _ = oracle.rerope_full(q1, q2, k1, k2, v, causal, 0.5, W)
+    out = triton_fused_attn_rerope.attention(q1.cuda(), q2.cuda(), k1.cuda(), k2.cuda(), v.cuda(), causal, 0.5, W)
+    torch.cuda.synchronize()
+    assert out.shape == q1.shape
+    assert (out.float().cpu() - want).abs().max() <= 2e-2
+    assert_close_16(out, want, "rerope_full")
+
+
+# ------------------------------------------------------------------ VQ prefill (additive codes)
+def _codes(B, H, N, M, K=256, seed=0):
+    g = torch.Generator("cpu").manual_seed(seed)
+    return torch.randint(0, K, (B, H, N, M), generator=g, dtype=torch.int32).to(torch.uint8)
+
+
+@pytest.mark.parametrize("B,H,N,D,M,K", [(1, 2, 1024, 64, 2, 256), (2, 2, 300, 128, 4, 256), (1, 1, 130, 128, 1, 64),
+                                          (1, 2, 777, 64, 8, 256), (1, 1, 64, 128, 4, 256)])
+@pytest.mark.parametrize("causal", [True, False])
+def test_vq_prefill_all_quantised(B, H, N, D, M, K, causal):
+    _say(f"vq prefill far-only B{B} H{H} N{N} D{D} M{M} K{K} causal={causal}")
+    q, v = _randn(B, H, N, D, seed=40), _randn(B, H, N, D, seed=41)
+    cb = _randn(H, M, K, D, seed=42, std=0.5 / math.sqrt(M))
+    codes = _codes(B, H, N, M, K, seed=43)
+    want, want_lse = oracle.attn_vq_prefill(q, codes, cb, v, causal=causal)
+    out, lse = attn_vq_prefill(q.cuda(), codes.cuda(), cb.cuda(), v.cuda(), causal=causal, return_lse=True)
+    torch.cuda.synchronize()
+    assert_close_16(out, want, "vq prefill")
+    assert_close_lse(lse, want_lse, atol=1e-2)  # far keys are rounded once to 16 bits before the dot product
+
+
+@pytest.mark.parametrize("boundary_mode", ["block", "exact"])
+@pytest.mark.parametrize("with_rerope", [False, True])
+@pytest.mark.parametrize("B,H,N,D,M,W", [(1, 2, 1024, 128, 4, 256), (2, 2, 640, 64, 2, 128), (1, 2, 515, 128, 4, 128),
+                                          (1, 1, 300, 128, 4, 384), (1, 2, 900, 128, 1, 200)])
+def test_vq_prefill_with_exact_window(B, H, N, D, M, W, with_rerope, boundary_mode):
+    _say(f"vq prefill window B{B} H{H} N{N} D{D} M{M} W{W} rerope={with_rerope} {boundary_mode}")
+    q, k, v, q2, k2 = (_randn(B, H, N, D, seed=50 + s) for s in range(5))
+    cb = _randn(H, M, 256, D, seed=55, std=0.35)
+    codes = _codes(B, H, N, M, seed=56)
+    kw = dict(k_exact=k, window_size=W, boundary_mode=boundary_mode)
+    if with_rerope:
+        kw.update(q2=q2, k2=k2)
+    want, want_lse = oracle.attn_vq_prefill(q, codes, cb, v, **kw)
+    kw = {n: (t.cuda() if torch.is_tensor(t) else t) for n, t in kw.items()}
+    out, lse = attn_vq_prefill(q.cuda(), codes.cuda(), cb.cuda(), v.cuda(), return_lse=True, **kw)
+    torch.cuda.synchronize()
+    assert_close_16(out, want, "vq prefill window")
+    assert_close_lse(lse, want_lse, atol=1e-2)
+
+
+def test_vq_prefill_far_boundary_is_exact():
+    """Mask/source check with little rounding slack: far keys score 1 (weight e), exact keys score 0 (weight 1), V rows
+    are position markers; a key taken from the wrong side moves its output element by ~1e-3, rounding by ~1e-5."""
+    N, D, W = 640, 128, 128
+    q = torch.zeros(1, 1, N, D, dtype=torch.bfloat16)
+    q[..., 0] = 1.0
+    cb = torch.zeros(1, 1, 256, D, dtype=torch.bfloat16)
+    cb[0, 0, :, 0] = 1.0
+    codes = torch.zeros(1, 1, N, 1, dtype=torch.uint8)
+    k = torch.zeros(1, 1, N, D, dtype=torch.bfloat16)
+    v = torch.zeros(1, 1, N, D, dtype=torch.bfloat16)
+    v[0, 0, torch.arange(N), torch.arange(N) % D] = 1.0
+    for bm in ("block", "exact"):
+        want, _ = oracle.attn_vq_prefill(q, codes, cb, v, k_exact=k, window_size=W, boundary_mode=bm, softmax_scale=1.0)
+        out = attn_vq_prefill(q.cuda(), codes.cuda(), cb.cuda(), v.cuda(), k_exact=k.cuda(), window_size=W,
+                              boundary_mode=bm, softmax_scale=1.0)
+        assert torch.allclose(out.float().cpu(), want, atol=1e-4, rtol=1e-2), bm
+
+
+# ------------------------------------------------------------------ reference-shaped single-codebook route
+def _count_route_case(N, W, C, D, H=2, B=1, dtype=torch.float16, seed=60):
+    q, k, v = (_randn(B, H, N, D, seed=seed + s, dtype=dtype) for s in range(3))
+    cb = _randn(H, C, D, seed=seed + 3, dtype=dtype)
+    cos, sin = oracle.rope_tables(D, N + W + 2)
+    pos = torch.arange(N)
+    q1, k1 = oracle.apply_rope(q, cos, sin, pos), oracle.apply_rope(k, cos, sin, pos)
+    q2 = oracle.apply_rope(q, cos, sin, W + 1)
+    k_hat, ids, _ = oracle.multi_head_single_quantize(k, cb)
+    cnt, v_vq, vi = oracle.sort_based_preprocess(ids, v, C, dtype=dtype)
+    return q1, q2, k1, k, k_hat, ids, cb, v, cnt.to(dtype), v_vq, vi
+
+
+@pytest.mark.parametrize("N,W,C,D", [(511, 256, 128, 64), (1024, 256, 256, 128), (900, 128, 512, 128)])
+def test_vq_attn_forward_reference_route(N, W, C, D):
+    """vq_attn_forward on inputs built by the sort-based preprocessing, against the naive per-key oracle (includes
+    the reference's own check shape: LEN=511, W=256, fp16, 2 heads of dim 64, ops/attn_vq.py:534-556)."""
+    _say(f"vq_attn_forward N{N} W{W} C{C} D{D}")
+    q1, q2, k1, k, k_hat, ids, cb, v, cnt, v_vq, vi = _count_route_case(N, W, C, D)
+    want, _ = oracle.attn_vq_prefill(q1, ids[..., None], cb[:, None], v, k_exact=k1, window_size=W, q2=q2, k2=k)
+    dev = [t.cuda() for t in (q1, q2, k1, cb, cnt, k, v, v_vq, vi)]
+    out = triton_fused_vq_attn.vq_attn_forward(*dev, W)
+    torch.cuda.synchronize()
+    assert out.shape == q1.shape
+    # oracle of the same route (count kernel on the same 16-bit prefix sums) bounds the kernel error tightly ...
+    route = oracle.vq_attn_forward(q1, q2, k1, cb, cnt, k, v, v_vq, vi, W)
+    assert_close_16(out, route, "count route")
+    # ... and the per-key definition within the reference's own acceptance
+    assert_close_16(out, want, "count route vs per-key")
+
+
+def test_count_kernel_and_merge_separately():
+    N, W, C, D = 700, 128, 256, 128
+    q1, q2, k1, k, k_hat, ids, cb, v, cnt, v_vq, vi = _count_route_case(N, W, C, D, B=2, dtype=torch.bfloat16)
+    want_o, want_l = oracle.vq_count_forward(q2, cb, cnt, v_vq, vi, W)
+    o2, l2 = triton_fused_vq_attn.vq_count_forward(q2.cuda(), cb.cuda(), cnt.cuda(), v_vq.cuda(), vi.cuda(), W)
+    torch.cuda.synchronize()
+    assert_close_16(o2, want_o, "count kernel")
+    assert_close_lse(l2, want_l, atol=5e-3)
+    assert torch.isinf(l2[:, :, : W + 128]).all() and (o2[:, :, : W + 128] == 0).all()
+    # merge in flashinfer's [N, B*H, D] layout against the oracle merge
+    o1, l1 = oracle.local_attn(q1, k1, v, W, "rerope", None, q2=q2, k2=k)
+    B, H = q1.shape[:2]
+    a = o1.to(torch.bfloat16).reshape(B * H, N, D).transpose(0, 1).contiguous().cuda()
+    sa = l1.reshape(B * H, N).transpose(0, 1).contiguous().cuda()
+    b = o2.reshape(B * H, N, D).transpose(0, 1).contiguous()
+    sb = l2.reshape(B * H, N).transpose(0, 1).contiguous()
+    want_m, want_s = oracle.merge_state(a, sa, b, sb)
+    triton_fused_vq_attn.merge_state_in_place(a, sa, b, sb)
+    torch.cuda.synchronize()
+    assert_close_16(a, want_m, "merge")
+    assert_close_lse(sa, want_s)

@@ -19,6 +19,17 @@ SIGNATURES = {
     "vqa_decode_workspace_bytes": (c_size_t, [c_int] * 7),
     "vqa_decode_bf16": (c_int, [_P] * 7 + [c_size_t] + [c_int] * 6 + [_STRIDES, c_float, c_int, _P]),
     "vqa_decode_f16": (c_int, [_P] * 7 + [c_size_t] + [c_int] * 6 + [_STRIDES, c_float, c_int, _P]),
+    "vqa_local_attn_bf16": (c_int, [_P] * 7 + [c_int] * 4 + [_STRIDES, c_int, c_int, c_float, _P]),
+    "vqa_local_attn_f16": (c_int, [_P] * 7 + [c_int] * 4 + [_STRIDES, c_int, c_int, c_float, _P]),
+    "vqa_rerope_full_bf16": (c_int, [_P] * 7 + [c_int] * 4 + [_STRIDES, c_int, c_int, c_float, _P]),
+    "vqa_rerope_full_f16": (c_int, [_P] * 7 + [c_int] * 4 + [_STRIDES, c_int, c_int, c_float, _P]),
+    "vqa_prefill_workspace_bytes": (c_size_t, [c_int] * 4),
+    "vqa_prefill_bf16": (c_int, [_P] * 10 + [c_size_t] + [c_int] * 6 + [_STRIDES, c_int, c_int, c_int, c_float, _P]),
+    "vqa_prefill_f16": (c_int, [_P] * 10 + [c_size_t] + [c_int] * 6 + [_STRIDES, c_int, c_int, c_int, c_float, _P]),
+    "vqa_vqcount_fwd_bf16": (c_int, [_P] * 7 + [c_int] * 5 + [_STRIDES, c_int, c_float, _P]),
+    "vqa_vqcount_fwd_f16": (c_int, [_P] * 7 + [c_int] * 5 + [_STRIDES, c_int, c_float, _P]),
+    "vqa_merge_state_inplace_bf16": (c_int, [_P] * 4 + [c_int] * 4 + [_STRIDES, _P]),
+    "vqa_merge_state_inplace_f16": (c_int, [_P] * 4 + [c_int] * 4 + [_STRIDES, _P]),
 }
 
 

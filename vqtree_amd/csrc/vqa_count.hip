@@ -1,0 +1,250 @@
+// Count-weighted softmax over codewords (single-codebook far context) and the base-2 log-sum-exp state merge.
+//
+// count kernel: query tile t covers rows [W + T + t*T, W + T + (t+1)*T) and attends over the C codewords of its
+// head: score_c = q2 . codebook[c]; codewords that no key up to block t uses (cnt == 0) are masked; the numerator
+// sums P . v_vq[vi[t, c]] (per-code running sums of V), the denominator weights exp by cnt[t, c].
+#include "vqa_flash.h"
+
+namespace vqa {
+namespace flash {
+
+struct CountParams {
+    View q;                 // q2 [B,H,N,D]
+    const uint16_t* cb;     // [H,C,D]
+    int64_t cb_sh, cb_sc;
+    const uint16_t* cnt;    // [B,H,NT,C] in the element type
+    int64_t cnt_sb, cnt_sh, cnt_st;
+    View vvq;               // [B,H,N+1,D]
+    const int64_t* vi;      // [B,H,NT,C]
+    int64_t vi_sb, vi_sh, vi_st;
+    uint16_t* out;
+    int64_t o_sb, o_sh, o_sn;
+    float* lse;             // [B,H,N]
+    int H, N, C, window, n_far_tiles;
+    float scale_log2e;
+};
+
+template <typename Tag, int D>
+__global__ __launch_bounds__(kThreads, 2) void count_kernel(CountParams p) {
+    typedef Geom<D> G;
+    typedef typename Elem<Tag>::vec8 vec8;
+    __shared__ __attribute__((aligned(16))) char s_k[G::kTileBytes];
+    __shared__ __attribute__((aligned(16))) char s_v[G::kTileBytes];
+    __shared__ float s_cnt[kBN];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int half = lane >> 5;
+    const int bh = blockIdx.y;
+    const int b = bh / p.H, h = bh % p.H;
+    uint16_t* out_base = p.out + b * p.o_sb + h * p.o_sh;
+    float* lse_base = p.lse ? p.lse + (int64_t)bh * p.N : nullptr;
+    const int first = p.window + kTile;  // first row with a far context
+
+    if ((int)blockIdx.x >= p.n_far_tiles) {
+        // rows [0, W+T): no far context -> out = 0, lse = -inf
+        const int m0 = ((int)blockIdx.x - p.n_far_tiles) * kBM;
+        const int rows = min(min(first, p.N) - m0, kBM);
+        for (int i = tid; i < rows * (D / 4); i += kThreads) {
+            const int r = i / (D / 4), c = i % (D / 4);
+            *reinterpret_cast<uint2*>(out_base + (int64_t)(m0 + r) * p.o_sn + c * 4) = make_uint2(0u, 0u);
+        }
+        if (lse_base)
+            for (int r = tid; r < rows; r += kThreads) lse_base[m0 + r] = -INFINITY;
+        return;
+    }
+
+    const int t = blockIdx.x;
+    const int row0 = first + t * kTile + wave * 32;
+    const uint16_t* cb = p.cb + h * p.cb_sh;
+    const uint16_t* cnt = p.cnt + b * p.cnt_sb + h * p.cnt_sh + t * p.cnt_st;
+    const int64_t* vi = p.vi + b * p.vi_sb + h * p.vi_sh + t * p.vi_st;
+    const uint16_t* vvq = p.vvq.p + b * p.vvq.sb + h * p.vvq.sh;
+
+    QFrag<Tag, D> q;
+    load_q<Tag, D>(q, p.q.p + b * p.q.sb + h * p.q.sh, p.q.sn, row0, p.N, lane);
+    SoftmaxState<D> st;
+    st.init();
+
+    for (int c0 = 0; c0 < p.C; c0 += kBN) {
+        TileRegs<D> kreg, vreg;
+        tile_g2r<D>(kreg, cb, p.cb_sc, c0, p.C, tid);
+        tile_g2r_gather<D>(vreg, vvq, p.vvq.sn, vi, c0, p.C, tid);
+        float cnt_f = 0.f;
+        if (tid < kBN && c0 + tid < p.C) cnt_f = Elem<Tag>::from_bits(cnt[c0 + tid]);
+        __syncthreads();  // previous tile fully consumed
+        tile_r2s<D>(kreg, s_k, tid);
+        tile_r2s<D>(vreg, s_v, tid);
+        if (tid < kBN) s_cnt[tid] = cnt_f;  // 0 for codewords past C: masked below
+        __syncthreads();
+
+        f32x16_t s[2];
+        qk_mma<Tag, D>(s, q, s_k, lane);
+        float w[2][16];
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float c = s_cnt[kb * 32 + key_of_reg(r, half)];
+                w[kb][r] = c;
+                s[kb][r] = (c != 0.f) ? s[kb][r] * p.scale_log2e : -INFINITY;
+            }
+        vec8 pf[2][2];
+        softmax_update<Tag, D, true>(st, s, pf, w);
+        pv_mma<Tag, D>(st.o, pf, s_v, lane);
+    }
+    store_output<Tag, D>(st, out_base, p.o_sn, lse_base, row0, p.N, lane);
+}
+
+// strides: q2(b,h,n) k_vq(h,c) k_vq_cnt(b,h,t) v_vq(b,h,n) vi(b,h,t) out(b,h,n)
+template <typename Tag>
+int vqcount(const void* q2, const void* k_vq, const void* k_vq_cnt, const void* v_vq, const int64_t* vi, void* out,
+            float* lse, int B, int H, int N, int D, int C, const int64_t* strides, int window, float sm_scale,
+            hipStream_t stream) {
+    if (!q2 || !k_vq || !k_vq_cnt || !v_vq || !vi || !out || !strides) return VQA_ERR_NULL_POINTER;
+    if (B <= 0 || H <= 0 || N <= 0 || C <= 0) return VQA_ERR_BAD_SHAPE;
+    if (window < 0 || (int64_t)B * H > 65535) return VQA_ERR_BAD_ARGUMENT;
+    CountParams p;
+    p.q = View{static_cast<const uint16_t*>(q2), strides[0], strides[1], strides[2]};
+    p.cb = static_cast<const uint16_t*>(k_vq);
+    p.cb_sh = strides[3], p.cb_sc = strides[4];
+    p.cnt = static_cast<const uint16_t*>(k_vq_cnt);
+    p.cnt_sb = strides[5], p.cnt_sh = strides[6], p.cnt_st = strides[7];
+    p.vvq = View{static_cast<const uint16_t*>(v_vq), strides[8], strides[9], strides[10]};
+    p.vi = vi;
+    p.vi_sb = strides[11], p.vi_sh = strides[12], p.vi_st = strides[13];
+    p.out = static_cast<uint16_t*>(out);
+    p.o_sb = strides[14], p.o_sh = strides[15], p.o_sn = strides[16];
+    p.lse = lse;
+    p.H = H, p.N = N, p.C = C, p.window = window;
+    p.scale_log2e = sm_scale * kLog2e;
+    if (!aligned16(p.q.p) || !aligned16(p.cb) || !aligned16(p.vvq.p) || ((uintptr_t)p.out & 7))
+        return VQA_ERR_MISALIGNED;
+    if (((p.q.sb | p.q.sh | p.q.sn | p.cb_sh | p.cb_sc | p.vvq.sb | p.vvq.sh | p.vvq.sn) & 7) ||
+        ((p.o_sb | p.o_sh | p.o_sn) & 3))
+        return VQA_ERR_MISALIGNED;
+    const int first = window + kTile;
+    p.n_far_tiles = N > first ? (N - first + kTile - 1) / kTile : 0;
+    const int zero_tiles = ((first < N ? first : N) + kBM - 1) / kBM;
+    const dim3 grid(p.n_far_tiles + zero_tiles, B * H);
+    if (D == 64)
+        hipLaunchKernelGGL((count_kernel<Tag, 64>), grid, dim3(kThreads), 0, stream, p);
+    else if (D == 128)
+        hipLaunchKernelGGL((count_kernel<Tag, 128>), grid, dim3(kThreads), 0, stream, p);
+    else
+        return VQA_ERR_UNSUPPORTED_HEAD_DIM;
+    return launch_status();
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// merge: (o, s) <- merge((o, s), (o', s')) with base-2 log-sum-exp s; one thread per 4 output elements.
+// ---------------------------------------------------------------------------------------------------------------
+struct MergeParams {
+    uint16_t* o;
+    int64_t o_sb, o_sh, o_sn;
+    float* s;
+    int64_t s_sb, s_sh, s_sn;
+    const uint16_t* o2;
+    int64_t o2_sb, o2_sh, o2_sn;
+    const float* s2;
+    int64_t s2_sb, s2_sh, s2_sn;
+    int H, N, D;
+};
+
+template <typename Tag>
+__global__ __launch_bounds__(256) void merge_kernel(MergeParams p) {
+    const int cpr = p.D / 4;  // 4-element chunks per row
+    const int rows_per_block = 256 / cpr;
+    const int n = blockIdx.x * rows_per_block + threadIdx.x / cpr;
+    const int c = threadIdx.x % cpr;
+    const int bh = blockIdx.y;
+    const int b = bh / p.H, h = bh % p.H;
+    const bool active = n < p.N && (int)threadIdx.x < rows_per_block * cpr;
+    const int nn = active ? n : blockIdx.x * rows_per_block;  // inactive threads shadow the block's first row
+    float* sp = p.s + b * p.s_sb + h * p.s_sh + nn * p.s_sn;
+    const float s1 = *sp;
+    const float s2 = p.s2[b * p.s2_sb + h * p.s2_sh + nn * p.s2_sn];
+    const float m = fmaxf(s1, s2);
+    const float m_safe = (m == -INFINITY) ? 0.f : m;
+    const float w1 = fast_exp2(s1 - m_safe), w2 = fast_exp2(s2 - m_safe);
+    const float den = w1 + w2;
+    const float inv = den > 0.f ? 1.f / den : 0.f;
+    uint16_t* op = p.o + b * p.o_sb + h * p.o_sh + nn * p.o_sn + c * 4;
+    const uint16_t* op2 = p.o2 + b * p.o2_sb + h * p.o2_sh + nn * p.o2_sn + c * 4;
+    const uint2 a = *reinterpret_cast<const uint2*>(op);
+    const uint2 bb = *reinterpret_cast<const uint2*>(op2);
+    const uint32_t aw[2] = {a.x, a.y}, bw[2] = {bb.x, bb.y};
+    uint32_t rw[2];
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+        const float lo = (Elem<Tag>::from_bits((uint16_t)(aw[e] & 0xffffu)) * w1 +
+                          Elem<Tag>::from_bits((uint16_t)(bw[e] & 0xffffu)) * w2) * inv;
+        const float hi = (Elem<Tag>::from_bits((uint16_t)(aw[e] >> 16)) * w1 +
+                          Elem<Tag>::from_bits((uint16_t)(bw[e] >> 16)) * w2) * inv;
+        rw[e] = (uint32_t)Elem<Tag>::to_bits(lo) | ((uint32_t)Elem<Tag>::to_bits(hi) << 16);
+    }
+    if (active) *reinterpret_cast<uint2*>(op) = make_uint2(rw[0], rw[1]);
+    __syncthreads();  // every thread of the row has read s before it is rewritten
+    if (active && c == 0) *sp = den > 0.f ? m + fast_log2(den) : -INFINITY;
+}
+
+// strides: o(b,h,n) s(b,h,n) o_other(b,h,n) s_other(b,h,n)
+template <typename Tag>
+int merge(void* o, float* s, const void* o_other, const float* s_other, int B, int H, int N, int D,
+          const int64_t* strides, hipStream_t stream) {
+    if (!o || !s || !o_other || !s_other || !strides) return VQA_ERR_NULL_POINTER;
+    if (B <= 0 || H <= 0 || N <= 0) return VQA_ERR_BAD_SHAPE;
+    if (D < 4 || D > 1024 || (D & 3)) return VQA_ERR_UNSUPPORTED_HEAD_DIM;
+    if ((int64_t)B * H > 65535) return VQA_ERR_BAD_ARGUMENT;
+    MergeParams p;
+    p.o = static_cast<uint16_t*>(o);
+    p.o_sb = strides[0], p.o_sh = strides[1], p.o_sn = strides[2];
+    p.s = s;
+    p.s_sb = strides[3], p.s_sh = strides[4], p.s_sn = strides[5];
+    p.o2 = static_cast<const uint16_t*>(o_other);
+    p.o2_sb = strides[6], p.o2_sh = strides[7], p.o2_sn = strides[8];
+    p.s2 = s_other;
+    p.s2_sb = strides[9], p.s2_sh = strides[10], p.s2_sn = strides[11];
+    p.H = H, p.N = N, p.D = D;
+    if (((uintptr_t)o & 7) || ((uintptr_t)o_other & 7) ||
+        ((p.o_sb | p.o_sh | p.o_sn | p.o2_sb | p.o2_sh | p.o2_sn) & 3))
+        return VQA_ERR_MISALIGNED;
+    const int cpr = D / 4;
+    if (cpr > 256) return VQA_ERR_UNSUPPORTED_HEAD_DIM;
+    const int rows_per_block = 256 / cpr;
+    const dim3 grid((N + rows_per_block - 1) / rows_per_block, B * H);
+    hipLaunchKernelGGL((merge_kernel<Tag>), grid, dim3(256), 0, stream, p);
+    return launch_status();
+}
+
+}  // namespace flash
+}  // namespace vqa
+
+extern "C" {
+
+int vqa_vqcount_fwd_bf16(const void* q2, const void* k_vq, const void* k_vq_cnt, const void* v_vq, const int64_t* vi,
+                         void* out, float* lse, int B, int H, int N, int D, int C, const int64_t* strides, int window,
+                         float sm_scale, vqa_stream_t stream) {
+    return vqa::flash::vqcount<vqa::bf16_tag>(q2, k_vq, k_vq_cnt, v_vq, vi, out, lse, B, H, N, D, C, strides, window,
+                                              sm_scale, stream);
+}
+
+int vqa_vqcount_fwd_f16(const void* q2, const void* k_vq, const void* k_vq_cnt, const void* v_vq, const int64_t* vi,
+                        void* out, float* lse, int B, int H, int N, int D, int C, const int64_t* strides, int window,
+                        float sm_scale, vqa_stream_t stream) {
+    return vqa::flash::vqcount<vqa::f16_tag>(q2, k_vq, k_vq_cnt, v_vq, vi, out, lse, B, H, N, D, C, strides, window,
+                                             sm_scale, stream);
+}
+
+int vqa_merge_state_inplace_bf16(void* o, float* s, const void* o_other, const float* s_other, int B, int H, int N,
+                                 int D, const int64_t* strides, vqa_stream_t stream) {
+    return vqa::flash::merge<vqa::bf16_tag>(o, s, o_other, s_other, B, H, N, D, strides, stream);
+}
+
+int vqa_merge_state_inplace_f16(void* o, float* s, const void* o_other, const float* s_other, int B, int H, int N,
+                                int D, const int64_t* strides, vqa_stream_t stream) {
+    return vqa::flash::merge<vqa::f16_tag>(o, s, o_other, s_other, B, H, N, D, strides, stream);
+}
+
+}  // extern "C"

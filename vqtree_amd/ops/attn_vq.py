@@ -62,3 +62,51 @@ def attn_vq_decode(q, k_codes, codebooks, v, *, softmax_scale=None, return_lse=F
             )
         )  # fmt: skip
     return (out, lse) if return_lse else out
+
+
+def attn_vq_prefill(q, k_codes, codebooks, v, *, k_exact=None, window_size=0, causal=True, softmax_scale=None,
+                    return_lse=False, boundary_mode="block", q2=None, k2=None):
+    """Prefill attention (seqlen_q == seqlen_k) over additive-quantiser key codes, optionally with an exact window.
+
+    q, v [B,H,N,D] bf16/f16; k_codes [B,H,N,M] uint8; codebooks [H,M,K,D].  With `k_exact` [B,H,N,D]: keys
+    j >= boundary(i) are exact (score q.k_exact inside the window i - j <= window_size; the strip between boundary and
+    window uses q2.k2 when both are given), older keys use their reconstruction sum_m codebooks[h,m,code] scored
+    with q2 if given else q.  boundary(i) = max(0, floor((i - W)/128)*128) for boundary_mode "block" (the rule of
+    ops/attn_vq.py:311 and of the window kernel stages), max(0, i - W) for "exact".  One softmax over all visible
+    keys: the window and far parts are merged inside the kernel.  Returns out [B,H,N,D] (and base-2 lse [B,H,N]).
+    """
+    from ._common import BOUNDARY, bhn_strides, check_same_16bit, last_dim_contiguous, ptr
+
+    lib = _lib.load()
+    _lib.require_gpu(q, k_codes, codebooks, v, k_exact, q2, k2)
+    B, H, N, D = q.shape
+    M, K = k_codes.shape[3], codebooks.shape[2]
+    assert k_codes.shape == (B, H, N, M) and k_codes.dtype == torch.uint8
+    assert codebooks.shape == (H, M, K, D), "codebooks must be [H,M,K,D]"
+    assert v.shape == (B, H, N, D), "seqlen_q == seqlen_k prefill only"
+    assert causal or k_exact is None, "non-causal attention takes quantised keys only"
+    sfx = check_same_16bit(q, codebooks, v, k_exact, q2, k2)
+    q, codebooks, v, k_exact, q2, k2 = last_dim_contiguous(q, codebooks, v, k_exact, q2, k2)
+    if k_codes.stride(3) != 1 or k_codes.stride(2) != M:
+        k_codes = k_codes.contiguous()
+    softmax_scale = softmax_scale or 1.0 / math.sqrt(D)
+    out = torch.empty((B, H, N, D), dtype=q.dtype, device=q.device)
+    lse = torch.empty((B, H, N), dtype=torch.float32, device=q.device) if return_lse else None
+    ws_bytes = lib.vqa_prefill_workspace_bytes(B, H, N, D)
+    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
+    dummy = (0, 0, 0)
+    strides = _lib.strides_array(
+        *bhn_strides(q), k_codes.stride(0), k_codes.stride(1),
+        codebooks.stride(0), codebooks.stride(1), codebooks.stride(2), *bhn_strides(v),
+        *(bhn_strides(k_exact) if k_exact is not None else dummy),
+        *(bhn_strides(q2) if q2 is not None else dummy),
+        *(bhn_strides(k2) if k2 is not None else dummy),
+        *bhn_strides(out),
+    )
+    with torch.cuda.device(q.device):
+        rc = getattr(lib, "vqa_prefill_" + sfx)(
+            ptr(q), ptr(k_codes), ptr(codebooks), ptr(v), ptr(k_exact), ptr(q2), ptr(k2), ptr(out), ptr(lse),
+            ptr(workspace), ws_bytes, B, H, N, D, M, K, strides, int(window_size), BOUNDARY[boundary_mode],
+            1 if causal else 0, softmax_scale, _lib.current_stream(q.device))
+    _lib.check(rc)
+    return (out, lse) if return_lse else out
