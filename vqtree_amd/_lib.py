@@ -4,7 +4,8 @@ import os
 from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
 
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_PKG_DIR, "libvqattn_gfx950.so")
+# VQATTN_LIB points at an alternative build of the same ABI (kernel tuning experiments)
+LIB_PATH = os.environ.get("VQATTN_LIB") or os.path.join(_PKG_DIR, "libvqattn_gfx950.so")
 
 _lib = None
 

@@ -19,6 +19,7 @@ typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
 
@@ -53,6 +54,11 @@ struct Elem<bf16_tag> {
         return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, b), acc,
                                                false);
     }
+    // two fp32 -> packed pair (lo = a, hi = b), round to nearest even (v_cvt_pk_bf16_f32)
+    static __device__ __forceinline__ uint32_t pack2(float a, float b) {
+        const f32x2_t v = {a, b};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+    }
     static __device__ __forceinline__ f32x4_t mfma16(vec8 a, vec8 b, f32x4_t c) {
         return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
     }
@@ -72,6 +78,10 @@ struct Elem<f16_tag> {
     static __device__ __forceinline__ float from_bits(uint16_t b) { return (float)__builtin_bit_cast(_Float16, b); }
     static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float acc) {
         return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, a), __builtin_bit_cast(f16x2_t, b), acc, false);
+    }
+    static __device__ __forceinline__ uint32_t pack2(float a, float b) {
+        const f32x2_t v = {a, b};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2_t));
     }
     static __device__ __forceinline__ f32x4_t mfma16(vec8 a, vec8 b, f32x4_t c) {
         return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);

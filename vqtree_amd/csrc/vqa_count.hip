@@ -28,8 +28,8 @@ template <typename Tag, int D>
 __global__ __launch_bounds__(kThreads, 2) void count_kernel(CountParams p) {
     typedef Geom<D> G;
     typedef typename Elem<Tag>::vec8 vec8;
-    __shared__ __attribute__((aligned(16))) char s_k[G::kTileBytes];
-    __shared__ __attribute__((aligned(16))) char s_v[G::kTileBytes];
+    __shared__ __attribute__((aligned(1024))) char s_k[G::kTileBytes];
+    __shared__ __attribute__((aligned(1024))) char s_v[G::kTileBytes];
     __shared__ float s_cnt[kBN];
 
     const int tid = threadIdx.x;
@@ -67,16 +67,19 @@ __global__ __launch_bounds__(kThreads, 2) void count_kernel(CountParams p) {
     SoftmaxState<D> st;
     st.init();
 
+    TileCopy<D, false> k_copy;
+    TileCopy<D, true> v_copy;
+    k_copy.init(wave, lane);
+    v_copy.init(wave, lane);
+
     for (int c0 = 0; c0 < p.C; c0 += kBN) {
-        TileRegs<D> kreg, vreg;
-        tile_g2r<D>(kreg, cb, p.cb_sc, c0, p.C, tid);
-        tile_g2r_gather<D>(vreg, vvq, p.vvq.sn, vi, c0, p.C, tid);
         float cnt_f = 0.f;
         if (tid < kBN && c0 + tid < p.C) cnt_f = Elem<Tag>::from_bits(cnt[c0 + tid]);
         __syncthreads();  // previous tile fully consumed
-        tile_r2s<D>(kreg, s_k, tid);
-        tile_r2s<D>(vreg, s_v, tid);
+        k_copy.load(s_k, cb, p.cb_sc, c0, p.C);
+        v_copy.load_gather(s_v, vvq, p.vvq.sn, vi, c0, p.C);
         if (tid < kBN) s_cnt[tid] = cnt_f;  // 0 for codewords past C: masked below
+        wait_tile_loads();
         __syncthreads();
 
         f32x16_t s[2];
@@ -88,10 +91,10 @@ __global__ __launch_bounds__(kThreads, 2) void count_kernel(CountParams p) {
             for (int r = 0; r < 16; ++r) {
                 const float c = s_cnt[kb * 32 + key_of_reg(r, half)];
                 w[kb][r] = c;
-                s[kb][r] = (c != 0.f) ? s[kb][r] * p.scale_log2e : -INFINITY;
+                s[kb][r] = (c != 0.f) ? s[kb][r] : -INFINITY;
             }
         vec8 pf[2][2];
-        softmax_update<Tag, D, true>(st, s, pf, w);
+        softmax_update<Tag, D, true>(st, s, p.scale_log2e, pf, w);
         pv_mma<Tag, D>(st.o, pf, s_v, lane);
     }
     store_output<Tag, D>(st, out_base, p.o_sn, lse_base, row0, p.N, lane);
@@ -104,7 +107,7 @@ int vqcount(const void* q2, const void* k_vq, const void* k_vq_cnt, const void* 
             hipStream_t stream) {
     if (!q2 || !k_vq || !k_vq_cnt || !v_vq || !vi || !out || !strides) return VQA_ERR_NULL_POINTER;
     if (B <= 0 || H <= 0 || N <= 0 || C <= 0) return VQA_ERR_BAD_SHAPE;
-    if (window < 0 || (int64_t)B * H > 65535) return VQA_ERR_BAD_ARGUMENT;
+    if (window < 0 || !(sm_scale > 0.f) || (int64_t)B * H > 65535) return VQA_ERR_BAD_ARGUMENT;
     CountParams p;
     p.q = View{static_cast<const uint16_t*>(q2), strides[0], strides[1], strides[2]};
     p.cb = static_cast<const uint16_t*>(k_vq);

@@ -8,6 +8,11 @@
 // are per-lane scalars (plus one exchange with lane ^ 32), and the probabilities are already laid out as the B
 // operand of O^T[d, query] = V^T . P^T.  V^T fragments (8 keys for one d per lane) are read from the row-major V
 // tile in LDS with ds_read_b64_tr_b16.
+//
+// K / V tiles travel HBM/L2 -> LDS without touching registers (global_load_lds_dwordx4: lane l of a wave writes
+// 16 bytes at LDS base + 16*l).  The tiles are unpadded; bank conflicts are avoided by an XOR swizzle of the 16-byte
+// chunk index with a function of the row, applied on the global-address side of the copy and undone when the MFMA
+// operands are read.
 #pragma once
 
 #include "vqa_common.h"
@@ -18,10 +23,14 @@ namespace flash {
 constexpr int kBM = 128;      // query rows per workgroup
 constexpr int kBN = 64;       // keys per tile
 constexpr int kThreads = 256; // 4 waves
+constexpr int kWaves = 4;
 constexpr int kTile = 128;    // T: block granularity of the window / far-context boundary rules
 
 typedef short s16x4_t __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));  // native vector: stays in registers
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+typedef __attribute__((address_space(3))) void* lds_void_ptr;
+typedef const __attribute__((address_space(1))) void* global_void_ptr;
 
 struct View {  // [B,H,N,D] tensor with unit innermost stride, element strides
     const uint16_t* p;
@@ -30,12 +39,23 @@ struct View {  // [B,H,N,D] tensor with unit innermost stride, element strides
 
 template <int D>
 struct Geom {
-    static constexpr int kPitch = D * 2 + 32;              // LDS row pitch in bytes (row shift of 8 banks)
-    static constexpr int kTileBytes = kBN * kPitch;
-    static constexpr int kChunksPerRow = D / 8;            // 16-byte chunks
-    static constexpr int kChunks = kBN * kChunksPerRow / kThreads;  // per thread
-    static constexpr int kKSteps = D / 16;                 // 32x32x16 steps along head_dim
-    static constexpr int kDBlocks = D / 32;                // 32-row blocks of O^T
+    static constexpr int kRowBytes = D * 2;
+    static constexpr int kTileBytes = kBN * kRowBytes;
+    static constexpr int kChunksPerRow = D / 8;                 // 16-byte chunks per row
+    static constexpr int kRowsPerInstr = 64 / kChunksPerRow;    // rows one wave-wide 16-byte load covers
+    static constexpr int kRowsPerWave = kBN / kWaves;           // 16
+    static constexpr int kInstr = kRowsPerWave / kRowsPerInstr; // direct-to-LDS loads per wave and tile
+    static constexpr int kRowsPerBankCycle = 256 / kRowBytes;   // rows that share one sweep over the 64 banks
+    static constexpr int kKSteps = D / 16;                      // 32x32x16 steps along head_dim
+    static constexpr int kDBlocks = D / 32;                     // 32-row blocks of O^T
+
+    // chunk-index XOR of a K tile row: 16 consecutive rows read the same logical chunk (ds_read_b128)
+    static __device__ __forceinline__ int swz_k(int row) { return (row / kRowsPerBankCycle) % kChunksPerRow; }
+    // chunk-index XOR of a V tile row: 8 consecutive rows x 4 consecutive chunks are read together
+    // (ds_read_b64_tr_b16); even values only, so the two 8-byte halves of a chunk stay together
+    static __device__ __forceinline__ int swz_v(int row) {
+        return 2 * ((row / kRowsPerBankCycle) % (kChunksPerRow / 2));
+    }
 };
 
 // Q fragment of one wave: B operand of S^T = K.Q^T.  Lane (n = lane%32, half = lane/32) holds
@@ -56,65 +76,91 @@ __device__ __forceinline__ void load_q(QFrag<Tag, D>& q, const uint16_t* base, i
     for (int kk = 0; kk < Geom<D>::kKSteps; ++kk) q.f[kk] = *reinterpret_cast<const vec8*>(r + kk * 16);
 }
 
-// Tile staging: global -> registers (16-byte chunks, row clamped to the last valid row) -> LDS.
-template <int D>
-struct TileRegs {
-    u32x4_t c[Geom<D>::kChunks];
+// ---------------------------------------------------------------------------------------------------------------
+// Tile copy global -> LDS.  Wave w brings rows [16w, 16w+16) of the 64-row tile; one instruction covers
+// kRowsPerInstr rows: lane l lands at LDS chunk (row, l % kChunksPerRow) and therefore fetches the global chunk
+// (l % kChunksPerRow) ^ swizzle(row).
+// ---------------------------------------------------------------------------------------------------------------
+template <int D, bool kIsV>
+struct TileCopy {
+    int row_in_instr;  // row (within the kRowsPerInstr rows of one instruction) this lane lands in
+    int chunk;         // LDS chunk column of this lane
+    int lds_wave_off;  // byte offset of the wave's first row inside the tile
+    int wave;
+
+    __device__ __forceinline__ void init(int wave_, int lane) {
+        wave = wave_;
+        row_in_instr = lane / Geom<D>::kChunksPerRow;
+        chunk = lane % Geom<D>::kChunksPerRow;
+        lds_wave_off = wave * Geom<D>::kRowsPerWave * Geom<D>::kRowBytes;
+    }
+    __device__ __forceinline__ int row(int i) const {
+        return wave * Geom<D>::kRowsPerWave + i * Geom<D>::kRowsPerInstr + row_in_instr;
+    }
+    __device__ __forceinline__ int src_chunk(int r) const {
+        return chunk ^ (kIsV ? Geom<D>::swz_v(r) : Geom<D>::swz_k(r));
+    }
+    // rows [n0, n0+64) of a [n_rows, D] matrix with row stride sn (elements); rows past the end repeat the last row
+    __device__ __forceinline__ void load(char* lds_tile, const uint16_t* base, int64_t sn, int n0, int n_rows) const {
+#pragma unroll
+        for (int i = 0; i < Geom<D>::kInstr; ++i) {
+            const int r = row(i);
+            const int g = min(n0 + r, n_rows - 1);
+            const uint16_t* src = base + (int64_t)g * sn + src_chunk(r) * 8;
+            __builtin_amdgcn_global_load_lds((global_void_ptr)src, (lds_void_ptr)(lds_tile + lds_wave_off + i * 1024),
+                                             16, 0, 0);
+        }
+    }
+    // same with the global row taken from an index list
+    __device__ __forceinline__ void load_gather(char* lds_tile, const uint16_t* base, int64_t sn,
+                                                const int64_t* row_index, int n0, int n_rows) const {
+#pragma unroll
+        for (int i = 0; i < Geom<D>::kInstr; ++i) {
+            const int r = row(i);
+            const int64_t g = row_index[min(n0 + r, n_rows - 1)];
+            const uint16_t* src = base + g * sn + src_chunk(r) * 8;
+            __builtin_amdgcn_global_load_lds((global_void_ptr)src, (lds_void_ptr)(lds_tile + lds_wave_off + i * 1024),
+                                             16, 0, 0);
+        }
+    }
 };
 
-template <int D>
-__device__ __forceinline__ void tile_g2r(TileRegs<D>& r, const uint16_t* base, int64_t sn, int n0, int n_rows,
-                                         int tid) {
-#pragma unroll
-    for (int i = 0; i < Geom<D>::kChunks; ++i) {
-        const int ch = tid + i * kThreads;
-        const int row = ch / Geom<D>::kChunksPerRow, col = ch % Geom<D>::kChunksPerRow;
-        const int g = min(n0 + row, n_rows - 1);
-        r.c[i] = *reinterpret_cast<const u32x4_t*>(base + (int64_t)g * sn + col * 8);
-    }
-}
-
-// Same, with the global row taken from an index list (rows of a gathered tensor).
-template <int D>
-__device__ __forceinline__ void tile_g2r_gather(TileRegs<D>& r, const uint16_t* base, int64_t sn,
-                                                const int64_t* row_index, int n0, int n_rows, int tid) {
-#pragma unroll
-    for (int i = 0; i < Geom<D>::kChunks; ++i) {
-        const int ch = tid + i * kThreads;
-        const int row = ch / Geom<D>::kChunksPerRow, col = ch % Geom<D>::kChunksPerRow;
-        const int64_t g = row_index[min(n0 + row, n_rows - 1)];
-        r.c[i] = *reinterpret_cast<const u32x4_t*>(base + g * sn + col * 8);
-    }
-}
-
-template <int D>
-__device__ __forceinline__ void tile_r2s(const TileRegs<D>& r, char* lds, int tid) {
-#pragma unroll
-    for (int i = 0; i < Geom<D>::kChunks; ++i) {
-        const int ch = tid + i * kThreads;
-        const int row = ch / Geom<D>::kChunksPerRow, col = ch % Geom<D>::kChunksPerRow;
-        *reinterpret_cast<u32x4_t*>(lds + row * Geom<D>::kPitch + col * 16) = r.c[i];
-    }
-}
+// all of this wave's direct-to-LDS loads have landed
+__device__ __forceinline__ void wait_tile_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 // S^T (64 keys x 32 queries) = Ktile . Q^T.  s[kb] is the accumulator of key block kb (32 keys); in it lane
 // (n, half) holds, at register r, key  kb*32 + 8*(r/4) + 4*half + r%4  of query n.
+// The A fragments are software-pipelined kAhead steps in front of their MFMA; the scheduling barriers pin that order
+// so only kAhead + 1 fragments are ever live (left alone, the scheduler hoists every LDS read to the top).
 template <typename Tag, int D>
 __device__ __forceinline__ void qk_mma(f32x16_t (&s)[2], const QFrag<Tag, D>& q, const char* lds_k, int lane) {
     typedef typename Elem<Tag>::vec8 vec8;
+    typedef Geom<D> G;
+    constexpr int KS = G::kKSteps;
+    constexpr int kSteps = 2 * KS;
+    constexpr int kAhead = 3;
     const int r = lane & 31, half = lane >> 5;
+    // logical chunk of step kk is 2*kk + half = (2*kk) ^ half; it is stored at chunk ^ swz_k(row), and
+    // swz_k(r) == swz_k(r + 32), so one per-lane base serves both key blocks
+    const uint32_t base = (uint32_t)(r * G::kRowBytes) | (uint32_t)((half ^ G::swz_k(r)) << 4);
+    auto frag = [&](int n) {
+        const uint32_t off = (base ^ (uint32_t)((2 * (n % KS)) << 4)) + (n / KS) * 32 * G::kRowBytes;
+        return *reinterpret_cast<const vec8*>(lds_k + off);
+    };
+    vec8 a[kAhead + 1];
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
-        f32x16_t acc;
+    for (int i = 0; i < kAhead; ++i) a[i] = frag(i);
+    f32x16_t acc;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) acc[i] = 0.f;
-        const char* row = lds_k + (kb * 32 + r) * Geom<D>::kPitch + half * 16;
+    for (int i = 0; i < kSteps; ++i) {
+        if (i + kAhead < kSteps) a[(i + kAhead) % (kAhead + 1)] = frag(i + kAhead);
+        if (i % KS == 0) {
 #pragma unroll
-        for (int kk = 0; kk < Geom<D>::kKSteps; ++kk) {
-            const vec8 a = *reinterpret_cast<const vec8*>(row + kk * 32);
-            acc = Elem<Tag>::mfma32(a, q.f[kk], acc);
+            for (int e = 0; e < 16; ++e) acc[e] = 0.f;
         }
-        s[kb] = acc;
+        acc = Elem<Tag>::mfma32(a[i % (kAhead + 1)], q.f[i % KS], acc);
+        if (i % KS == KS - 1) s[i / KS] = acc;
+        __builtin_amdgcn_sched_barrier(0);
     }
 }
 
@@ -124,32 +170,41 @@ __device__ __forceinline__ int key_of_reg(int r, int half) { return 8 * (r >> 2)
 // O^T (D x 32 queries) += Vtile^T . P^T.  p[kb][j2] packs the probabilities of keys kb*32 + j2*16 + {4*half..+3,
 // 8+4*half..+3} (registers j2*8 .. j2*8+7 of s[kb]) as the B operand; the matching V^T A operand is gathered by two
 // transposing LDS reads: inside every 16-lane group, source lane s points at V[key0 + s/4][d0 + 4*(s%4)] and lane L
-// receives V[key0 .. key0+3][d0 + L].
+// receives V[key0 .. key0+3][d0 + L].  Pipelined like qk_mma.
 template <typename Tag, int D>
 __device__ __forceinline__ void pv_mma(f32x16_t (&o)[Geom<D>::kDBlocks], const typename Elem<Tag>::vec8 (&p)[2][2],
                                        const char* lds_v, int lane) {
     typedef typename Elem<Tag>::vec8 vec8;
     typedef __attribute__((address_space(3))) s16x4_t* lds_ptr_t;
+    typedef Geom<D> G;
+    constexpr int DB = G::kDBlocks;
+    constexpr int kSteps = 4 * DB;  // (kb, j2, db)
+    constexpr int kAhead = 3;
     const int half = lane >> 5;
     const int dsub = (lane >> 4) & 1;  // which 16 of the 32 d rows this 16-lane group produces
-    const int s = lane & 15;
-    // address of this lane's 4-element source chunk for key0 = 0, d block 0
-    const char* src = lds_v + (4 * half + (s >> 2)) * Geom<D>::kPitch + (dsub * 16 + 4 * (s & 3)) * 2;
+    const int sl = lane & 15;
+    // source of this lane for key0 = 0, d block 0: row 4*half + sl/4, elements d = dsub*16 + 4*(sl%4) .. +3, i.e.
+    // logical chunk 2*dsub + (sl%4)/2, 8-byte piece (sl%4)%2.  Rows advance by multiples of 8, which leaves swz_v
+    // unchanged; d block db adds 4*db to the chunk, an XOR because the lane part only uses bits 0-1.
+    const int row = 4 * half + (sl >> 2);
+    const uint32_t base = (uint32_t)(row * G::kRowBytes) |
+                          (uint32_t)(((2 * dsub + ((sl & 3) >> 1)) ^ G::swz_v(row)) << 4) | (uint32_t)((sl & 1) << 3);
+    s16x4_t lo[kAhead + 1], hi[kAhead + 1];
+    auto fetch = [&](int n) {
+        const uint32_t off = (base ^ (uint32_t)((4 * (n % DB)) << 4)) + (n / DB) * 16 * G::kRowBytes;
+        lo[n % (kAhead + 1)] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr_t)(lds_v + off));
+        hi[n % (kAhead + 1)] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr_t)(lds_v + off + 8 * G::kRowBytes));
+    };
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
+    for (int i = 0; i < kAhead; ++i) fetch(i);
 #pragma unroll
-        for (int j2 = 0; j2 < 2; ++j2) {
-            const char* kbase = src + (kb * 32 + j2 * 16) * Geom<D>::kPitch;
-#pragma unroll
-            for (int db = 0; db < Geom<D>::kDBlocks; ++db) {
-                const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr_t)(kbase + db * 64));
-                const s16x4_t hi =
-                    __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr_t)(kbase + 8 * Geom<D>::kPitch + db * 64));
-                const short __attribute__((ext_vector_type(8))) av = {lo[0], lo[1], lo[2], lo[3],
-                                                                      hi[0], hi[1], hi[2], hi[3]};
-                o[db] = Elem<Tag>::mfma32(__builtin_bit_cast(vec8, av), p[kb][j2], o[db]);
-            }
-        }
+    for (int i = 0; i < kSteps; ++i) {
+        if (i + kAhead < kSteps) fetch(i + kAhead);
+        const s16x4_t l4 = lo[i % (kAhead + 1)], h4 = hi[i % (kAhead + 1)];
+        const short __attribute__((ext_vector_type(8))) av = {l4[0], l4[1], l4[2], l4[3], h4[0], h4[1], h4[2], h4[3]};
+        const int kbj = i / DB;  // kb*2 + j2
+        o[i % DB] = Elem<Tag>::mfma32(__builtin_bit_cast(vec8, av), p[kbj >> 1][kbj & 1], o[i % DB]);
+        __builtin_amdgcn_sched_barrier(0);
     }
 }
 
@@ -169,10 +224,12 @@ struct SoftmaxState {
     }
 };
 
-// s holds scaled (base-2) scores with masked entries at -inf; w (nullable per-register weights) multiplies the
-// probabilities in the row sum only (count-weighted softmax).  Produces the packed P^T fragments.
+// s holds RAW scores (masked entries at -inf); scale = sm_scale*log2(e) > 0 is folded into the exponent:
+// p = 2^(s*scale - m).  w (nullable per-register weights) multiplies the probabilities in the row sum only
+// (count-weighted softmax).  O is rescaled only when some row of the wave raised its maximum.  Produces the packed
+// P^T fragments.
 template <typename Tag, int D, bool kWeighted>
-__device__ __forceinline__ void softmax_update(SoftmaxState<D>& st, f32x16_t (&s)[2],
+__device__ __forceinline__ void softmax_update(SoftmaxState<D>& st, f32x16_t (&s)[2], float scale,
                                                typename Elem<Tag>::vec8 (&p)[2][2], const float (*w)[16]) {
     float mx = -INFINITY;
 #pragma unroll
@@ -180,34 +237,38 @@ __device__ __forceinline__ void softmax_update(SoftmaxState<D>& st, f32x16_t (&s
 #pragma unroll
         for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[kb][i]);
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float m_new = fmaxf(st.m, mx);
+    const float m_new = fmaxf(st.m, mx * scale);
     const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;  // a row with nothing visible yet keeps p = 0
-    const float alpha = fast_exp2(st.m - m_safe);
+    if (__builtin_amdgcn_ballot_w64(m_new != st.m) != 0) {
+        const float alpha = fast_exp2(st.m - m_safe);
+        st.l *= alpha;
+#pragma unroll
+        for (int db = 0; db < Geom<D>::kDBlocks; ++db)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) st.o[db][i] *= alpha;
+        st.m = m_new;
+    }
     float sum = 0.f;
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
         for (int j2 = 0; j2 < 2; ++j2) {
-            short __attribute__((ext_vector_type(8))) pk;
+            u32x4_t pk;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const int r = j2 * 8 + e;
-                const float pe = fast_exp2(s[kb][r] - m_safe);
+            for (int e = 0; e < 4; ++e) {
+                const int r = j2 * 8 + 2 * e;
+                const float p0 = fast_exp2(__builtin_fmaf(s[kb][r], scale, -m_safe));
+                const float p1 = fast_exp2(__builtin_fmaf(s[kb][r + 1], scale, -m_safe));
                 if constexpr (kWeighted)
-                    sum += pe * w[kb][r];
+                    sum += p0 * w[kb][r] + p1 * w[kb][r + 1];
                 else
-                    sum += pe;
-                pk[e] = (short)Elem<Tag>::to_bits(pe);
+                    sum += p0 + p1;
+                pk[e] = Elem<Tag>::pack2(p0, p1);
             }
             p[kb][j2] = __builtin_bit_cast(typename Elem<Tag>::vec8, pk);
         }
     }
-    st.l = st.l * alpha + sum;
-    st.m = m_new;
-#pragma unroll
-    for (int db = 0; db < Geom<D>::kDBlocks; ++db)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) st.o[db][i] *= alpha;
+    st.l += sum;
 }
 
 // Normalise and store the wave's 32 output rows; lse2 = m + log2(l).  A row that saw no key stores 0 / -inf.

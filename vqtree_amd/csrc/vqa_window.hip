@@ -115,17 +115,30 @@ __global__ __launch_bounds__(kThreads, 2) void window_kernel(Params p) {
     typedef typename Elem<Tag>::vec8 vec8;
     constexpr bool kDual = (MODE == kLocalRerope || MODE == kFullRerope || MODE == kVqPrefill);
 
-    __shared__ __attribute__((aligned(16))) char s_k[G::kTileBytes];
-    __shared__ __attribute__((aligned(16))) char s_k2[kDual ? G::kTileBytes : 16];
-    __shared__ __attribute__((aligned(16))) char s_v[G::kTileBytes];
+    // double-buffered K and V tiles, filled by direct global -> LDS loads one tile ahead of the compute
+    __shared__ __attribute__((aligned(1024))) char s_k[2][G::kTileBytes];
+    __shared__ __attribute__((aligned(1024))) char s_v[2][G::kTileBytes];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int half = lane >> 5, nq = lane & 31;
-    const int bh = blockIdx.y;
+    // Workgroups are dispatched round-robin over the 8 XCDs (each with its own L2) in linear-id order.  Give every
+    // XCD whole (batch, head) problems: the query tiles of one head then share its K/V through one L2.
+    int bh, t;
+    {
+        const int n_tiles = gridDim.x, n_bh = gridDim.y;
+        const int id = blockIdx.x + n_tiles * blockIdx.y;
+        if (n_bh % 8 == 0) {
+            const int xcd = id & 7, k = id >> 3;
+            bh = xcd + 8 * (k / n_tiles);
+            t = n_tiles - 1 - (k % n_tiles);  // long (late) query tiles first
+        } else {
+            bh = blockIdx.y;
+            t = n_tiles - 1 - blockIdx.x;
+        }
+    }
     const int b = bh / p.H, h = bh % p.H;
-    const int t = gridDim.x - 1 - blockIdx.x;  // long (late) query tiles are scheduled first
     const int m0 = t * kBM;
     const int m1 = min(m0 + kBM - 1, p.N - 1);
     const int row0 = m0 + wave * 32;
@@ -139,9 +152,23 @@ __global__ __launch_bounds__(kThreads, 2) void window_kernel(Params p) {
     auto k_ptr = [&](int src) { return src == 0 ? ka : (src == 1 ? kb_ : kc); };
     auto k_stride = [&](int src) { return src == 0 ? p.ka.sn : (src == 1 ? p.kb.sn : p.kc.sn); };
 
-    QFrag<Tag, D> qa, qb;
-    load_q<Tag, D>(qa, p.qa.p + b * p.qa.sb + h * p.qa.sh, p.qa.sn, row0, p.N, lane);
-    if constexpr (kDual) load_q<Tag, D>(qb, p.qb.p + b * p.qb.sb + h * p.qb.sh, p.qb.sn, row0, p.N, lane);
+    // One query fragment set lives in registers: pair A's or pair B's.  Tiles are visited far -> near, so the
+    // operand in use changes O(1) times per workgroup; a change re-reads the wave's 32 rows (L2 hits).
+    const uint16_t* qa_src = p.qa.p + b * p.qa.sb + h * p.qa.sh;
+    const uint16_t* qb_src = p.qb.p + b * p.qb.sb + h * p.qb.sh;
+    QFrag<Tag, D> q;
+    int q_held = -1;
+    auto hold_q = [&](int which) {  // which: 0 = qa, 1 = qb (workgroup-uniform)
+        if (q_held != which) {
+            load_q<Tag, D>(q, which == 0 ? qa_src : qb_src, which == 0 ? p.qa.sn : p.qb.sn, row0, p.N, lane);
+            q_held = which;
+        }
+    };
+
+    TileCopy<D, false> k_copy;
+    TileCopy<D, true> v_copy;
+    k_copy.init(wave, lane);
+    v_copy.init(wave, lane);
 
     // key tiles this workgroup visits
     const int hi_key = rules.is_causal() ? min(p.N, m1 + 1) : p.N;
@@ -151,52 +178,44 @@ __global__ __launch_bounds__(kThreads, 2) void window_kernel(Params p) {
     SoftmaxState<D> st;
     st.init();
 
-    TileRegs<D> kreg, vreg;
-#define VQA_PREFETCH(n0_)                                                                  \
-    do {                                                                                   \
-        const TileClass tn_ = classify<MODE>(rules, m0, m1, (n0_));                        \
-        tile_g2r<D>(kreg, k_ptr(tn_.main), k_stride(tn_.main), (n0_), p.N, tid);           \
-        tile_g2r<D>(vreg, v_src, p.v.sn, (n0_), p.N, tid);                                 \
-    } while (0)
-    VQA_PREFETCH(u_lo * kBN);
+    int buf = 0;  // buffer holding the tile about to be computed: K of its main pair, and V
+    {
+        const int src = classify<MODE>(rules, m0, m1, u_lo * kBN).main;
+        k_copy.load(s_k[0], k_ptr(src), k_stride(src), u_lo * kBN, p.N);
+        v_copy.load(s_v[0], v_src, p.v.sn, u_lo * kBN, p.N);
+    }
+
+    auto prefetch = [&](int n0_next, int into) {  // K of the tile's main pair + V, into buffer `into`
+        const int src = classify<MODE>(rules, m0, m1, n0_next).main;
+        k_copy.load(s_k[into], k_ptr(src), k_stride(src), n0_next, p.N);
+        v_copy.load(s_v[into], v_src, p.v.sn, n0_next, p.N);
+    };
 
     for (int u = u_lo; u < u_hi; ++u) {
         const int n0 = u * kBN;
         const bool more = u + 1 < u_hi;
-        __syncthreads();  // every wave has finished reading the previous tile
-        tile_r2s<D>(kreg, s_k, tid);
-        tile_r2s<D>(vreg, s_v, tid);
-        __syncthreads();
         const TileClass tc = classify<MODE>(rules, m0, m1, n0);
+        wait_tile_loads();
+        __syncthreads();  // tile u is complete in `buf`; every wave is done with the other buffer
+        hold_q(kDual && tc.main != 0 ? 1 : 0);
+        if (tc.fast && more) prefetch(n0 + kBN, buf ^ 1);  // next tile's loads fly while this one is computed
 
         f32x16_t s[2];
-        if (tc.fast) {
-            if (more) VQA_PREFETCH(n0 + kBN);  // next tile's loads fly while this one is computed
-            if constexpr (kDual) {
-                qk_mma<Tag, D>(s, tc.main == 0 ? qa : qb, s_k, lane);
-            } else {
-                qk_mma<Tag, D>(s, qa, s_k, lane);
-            }
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) s[kb][r] *= p.scale_log2e;
-        } else {
+        qk_mma<Tag, D>(s, q, s_k[buf], lane);
+        if (!tc.fast) {
+            // tile on the diagonal / window edge / far-context boundary: every pair it touches, per-element
+            // selection and masking
             const int qi = row0 + nq;
             if constexpr (kDual) {
-                qk_mma<Tag, D>(s, tc.main == 0 ? qa : qb, s_k, lane);
-                // the other pairs this tile touches, one K tile at a time through the second buffer
+                // the other pairs, one K tile at a time through the (still free) K buffer of the next tile
                 for (int src = 0; src < 3; ++src) {
                     if (src == tc.main || !((tc.need >> src) & 1)) continue;
-                    {
-                        TileRegs<D> k2;
-                        tile_g2r<D>(k2, k_ptr(src), k_stride(src), n0, p.N, tid);
-                        __syncthreads();  // previous readers of s_k2 are done
-                        tile_r2s<D>(k2, s_k2, tid);
-                    }
+                    k_copy.load(s_k[buf ^ 1], k_ptr(src), k_stride(src), n0, p.N);
+                    hold_q(src == 0 ? 0 : 1);
+                    wait_tile_loads();
                     __syncthreads();
                     f32x16_t s2[2];
-                    qk_mma<Tag, D>(s2, src == 0 ? qa : qb, s_k2, lane);
+                    qk_mma<Tag, D>(s2, q, s_k[buf ^ 1], lane);
 #pragma unroll
                     for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
@@ -204,26 +223,25 @@ __global__ __launch_bounds__(kThreads, 2) void window_kernel(Params p) {
                             const int j = n0 + kb * 32 + key_of_reg(r, half);
                             if (rules.source(qi, j) == src) s[kb][r] = s2[kb][r];
                         }
+                    __syncthreads();  // all waves have read this pair's K tile before the buffer is reused
                 }
-            } else {
-                qk_mma<Tag, D>(s, qa, s_k, lane);
             }
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int j = n0 + kb * 32 + key_of_reg(r, half);
-                    s[kb][r] = rules.visible(qi, j) ? s[kb][r] * p.scale_log2e : -INFINITY;
+                    s[kb][r] = rules.visible(qi, j) ? s[kb][r] : -INFINITY;
                 }
-            if (more) VQA_PREFETCH(n0 + kBN);
+            if (more) prefetch(n0 + kBN, buf ^ 1);
         }
 
         vec8 pf[2][2];
-        softmax_update<Tag, D, false>(st, s, pf, nullptr);
-        pv_mma<Tag, D>(st.o, pf, s_v, lane);
+        softmax_update<Tag, D, false>(st, s, p.scale_log2e, pf, nullptr);
+        pv_mma<Tag, D>(st.o, pf, s_v[buf], lane);
+        buf ^= 1;
     }
 
-#undef VQA_PREFETCH
     store_output<Tag, D>(st, p.out + b * p.o_sb + h * p.o_sh, p.o_sn,
                          p.lse ? p.lse + (int64_t)bh * p.N : nullptr, row0, p.N, lane);
 }
@@ -255,7 +273,7 @@ template <typename Tag>
 int run(Params p, int B, int D, int mode, hipStream_t stream) {
     if (B <= 0 || p.H <= 0 || p.N <= 0) return VQA_ERR_BAD_SHAPE;
     if ((int64_t)B * p.H > 65535) return VQA_ERR_BAD_ARGUMENT;
-    if (p.window < 0) return VQA_ERR_BAD_ARGUMENT;
+    if (p.window < 0 || !(p.scale_log2e > 0.f)) return VQA_ERR_BAD_ARGUMENT;
     if (!view_ok(p.qa) || !view_ok(p.qb) || !view_ok(p.ka) || !view_ok(p.kb) || !view_ok(p.kc) || !view_ok(p.v))
         return (p.qa.p && p.qb.p && p.ka.p && p.kb.p && p.kc.p && p.v.p) ? VQA_ERR_MISALIGNED : VQA_ERR_NULL_POINTER;
     if (!p.out) return VQA_ERR_NULL_POINTER;
