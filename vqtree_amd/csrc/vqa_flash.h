@@ -81,34 +81,62 @@ __device__ __forceinline__ void load_q(QFrag<Tag, D>& q, const uint16_t* base, i
 // kRowsPerInstr rows: lane l lands at LDS chunk (row, l % kChunksPerRow) and therefore fetches the global chunk
 // (l % kChunksPerRow) ^ swizzle(row).
 // ---------------------------------------------------------------------------------------------------------------
+// 16 bytes per lane from global memory straight into LDS: lane l of the wave lands at lds_addr + 16*l.
+// Issued as inline assembly on purpose: the compiler makes every later LDS read wait for all direct-to-LDS loads
+// it knows of (it cannot tell the buffer being filled from the one being read), which would serialise the
+// prefetch with the compute.  The kernels wait for these loads themselves (wait_tile_loads + barrier).
+__device__ __forceinline__ void dma16(const void* gptr, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                 :
+                 : "v"(gptr), "s"(lds_addr)
+                 : "memory");  // m0 is written too; no other instruction of these kernels uses it
+}
+
+__device__ __forceinline__ uint32_t lds_addr_of(const char* p) {
+    return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) char*)p;
+}
+
 template <int D, bool kIsV>
 struct TileCopy {
-    int row_in_instr;  // row (within the kRowsPerInstr rows of one instruction) this lane lands in
-    int chunk;         // LDS chunk column of this lane
-    int lds_wave_off;  // byte offset of the wave's first row inside the tile
     int wave;
+    int lane_row;                           // row (within the kRowsPerInstr rows of one instruction) of this lane
+    int chunk;                              // LDS chunk column of this lane
+    uint32_t chunk_bytes[Geom<D>::kInstr];  // byte offset inside the global row that lands in that column
 
     __device__ __forceinline__ void init(int wave_, int lane) {
         wave = wave_;
-        row_in_instr = lane / Geom<D>::kChunksPerRow;
+        lane_row = lane / Geom<D>::kChunksPerRow;
         chunk = lane % Geom<D>::kChunksPerRow;
-        lds_wave_off = wave * Geom<D>::kRowsPerWave * Geom<D>::kRowBytes;
+#pragma unroll
+        for (int i = 0; i < Geom<D>::kInstr; ++i) chunk_bytes[i] = (uint32_t)src_chunk(row(i)) * 16u;
     }
     __device__ __forceinline__ int row(int i) const {
-        return wave * Geom<D>::kRowsPerWave + i * Geom<D>::kRowsPerInstr + row_in_instr;
+        return wave * Geom<D>::kRowsPerWave + i * Geom<D>::kRowsPerInstr + lane_row;
     }
     __device__ __forceinline__ int src_chunk(int r) const {
         return chunk ^ (kIsV ? Geom<D>::swz_v(r) : Geom<D>::swz_k(r));
     }
+    __device__ __forceinline__ uint32_t dst(const char* lds_tile, int i) const {
+        return lds_addr_of(lds_tile) + (wave * Geom<D>::kRowsPerWave + i * Geom<D>::kRowsPerInstr) * Geom<D>::kRowBytes;
+    }
     // rows [n0, n0+64) of a [n_rows, D] matrix with row stride sn (elements); rows past the end repeat the last row
     __device__ __forceinline__ void load(char* lds_tile, const uint16_t* base, int64_t sn, int n0, int n_rows) const {
+        if (n0 + kBN <= n_rows) {
+            // uniform (scalar) tile/row-group base + one 32-bit per-lane offset
+            const uint32_t lane_off = (uint32_t)lane_row * (uint32_t)(sn * 2);
 #pragma unroll
-        for (int i = 0; i < Geom<D>::kInstr; ++i) {
-            const int r = row(i);
-            const int g = min(n0 + r, n_rows - 1);
-            const uint16_t* src = base + (int64_t)g * sn + src_chunk(r) * 8;
-            __builtin_amdgcn_global_load_lds((global_void_ptr)src, (lds_void_ptr)(lds_tile + lds_wave_off + i * 1024),
-                                             16, 0, 0);
+            for (int i = 0; i < Geom<D>::kInstr; ++i) {
+                const char* grp = reinterpret_cast<const char*>(
+                    base + (int64_t)(n0 + wave * Geom<D>::kRowsPerWave + i * Geom<D>::kRowsPerInstr) * sn);
+                dma16(grp + (lane_off + chunk_bytes[i]), dst(lds_tile, i));
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < Geom<D>::kInstr; ++i) {
+                const int g = min(n0 + row(i), n_rows - 1);
+                const char* src = reinterpret_cast<const char*>(base + (int64_t)g * sn) + chunk_bytes[i];
+                dma16(src, dst(lds_tile, i));
+            }
         }
     }
     // same with the global row taken from an index list
@@ -116,17 +144,16 @@ struct TileCopy {
                                                 const int64_t* row_index, int n0, int n_rows) const {
 #pragma unroll
         for (int i = 0; i < Geom<D>::kInstr; ++i) {
-            const int r = row(i);
-            const int64_t g = row_index[min(n0 + r, n_rows - 1)];
-            const uint16_t* src = base + g * sn + src_chunk(r) * 8;
-            __builtin_amdgcn_global_load_lds((global_void_ptr)src, (lds_void_ptr)(lds_tile + lds_wave_off + i * 1024),
-                                             16, 0, 0);
+            const int64_t g = row_index[min(n0 + row(i), n_rows - 1)];
+            const char* src = reinterpret_cast<const char*>(base + g * sn) + chunk_bytes[i];
+            dma16(src, dst(lds_tile, i));
         }
     }
 };
 
 // all of this wave's direct-to-LDS loads have landed
-__device__ __forceinline__ void wait_tile_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+// (s_waitcnt vmcnt(0) with expcnt / lgkmcnt left at their maxima)
+__device__ __forceinline__ void wait_tile_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }
 
 // S^T (64 keys x 32 queries) = Ktile . Q^T.  s[kb] is the accumulator of key block kb (32 keys); in it lane
 // (n, half) holds, at register r, key  kb*32 + 8*(r/4) + 4*half + r%4  of query n.
@@ -142,10 +169,13 @@ __device__ __forceinline__ void qk_mma(f32x16_t (&s)[2], const QFrag<Tag, D>& q,
     const int r = lane & 31, half = lane >> 5;
     // logical chunk of step kk is 2*kk + half = (2*kk) ^ half; it is stored at chunk ^ swz_k(row), and
     // swz_k(r) == swz_k(r + 32), so one per-lane base serves both key blocks
-    const uint32_t base = (uint32_t)(r * G::kRowBytes) | (uint32_t)((half ^ G::swz_k(r)) << 4);
+    // (the tile is 1 KiB-aligned in LDS, so the XOR may be applied to the full 32-bit LDS address)
+    typedef const __attribute__((address_space(3))) vec8* lds_vec8_ptr;
+    const uint32_t base = (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) char*)lds_k +
+                          ((uint32_t)(r * G::kRowBytes) | (uint32_t)((half ^ G::swz_k(r)) << 4));
     auto frag = [&](int n) {
-        const uint32_t off = (base ^ (uint32_t)((2 * (n % KS)) << 4)) + (n / KS) * 32 * G::kRowBytes;
-        return *reinterpret_cast<const vec8*>(lds_k + off);
+        const uint32_t addr = (base ^ (uint32_t)((2 * (n % KS)) << 4)) + (n / KS) * 32 * G::kRowBytes;
+        return *(lds_vec8_ptr)(uintptr_t)addr;
     };
     vec8 a[kAhead + 1];
 #pragma unroll
@@ -187,13 +217,15 @@ __device__ __forceinline__ void pv_mma(f32x16_t (&o)[Geom<D>::kDBlocks], const t
     // logical chunk 2*dsub + (sl%4)/2, 8-byte piece (sl%4)%2.  Rows advance by multiples of 8, which leaves swz_v
     // unchanged; d block db adds 4*db to the chunk, an XOR because the lane part only uses bits 0-1.
     const int row = 4 * half + (sl >> 2);
-    const uint32_t base = (uint32_t)(row * G::kRowBytes) |
-                          (uint32_t)(((2 * dsub + ((sl & 3) >> 1)) ^ G::swz_v(row)) << 4) | (uint32_t)((sl & 1) << 3);
+    const uint32_t base = (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) char*)lds_v +
+                          ((uint32_t)(row * G::kRowBytes) |
+                           (uint32_t)(((2 * dsub + ((sl & 3) >> 1)) ^ G::swz_v(row)) << 4) | (uint32_t)((sl & 1) << 3));
     s16x4_t lo[kAhead + 1], hi[kAhead + 1];
     auto fetch = [&](int n) {
-        const uint32_t off = (base ^ (uint32_t)((4 * (n % DB)) << 4)) + (n / DB) * 16 * G::kRowBytes;
-        lo[n % (kAhead + 1)] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr_t)(lds_v + off));
-        hi[n % (kAhead + 1)] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr_t)(lds_v + off + 8 * G::kRowBytes));
+        const uint32_t addr = (base ^ (uint32_t)((4 * (n % DB)) << 4)) + (n / DB) * 16 * G::kRowBytes;
+        lo[n % (kAhead + 1)] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr_t)(uintptr_t)addr);
+        hi[n % (kAhead + 1)] =
+            __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr_t)(uintptr_t)(addr + 8 * G::kRowBytes));
     };
 #pragma unroll
     for (int i = 0; i < kAhead; ++i) fetch(i);

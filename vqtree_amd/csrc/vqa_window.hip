@@ -161,6 +161,7 @@ __global__ __launch_bounds__(kThreads, 2) void window_kernel(Params p) {
     auto hold_q = [&](int which) {  // which: 0 = qa, 1 = qb (workgroup-uniform)
         if (q_held != which) {
             load_q<Tag, D>(q, which == 0 ? qa_src : qb_src, which == 0 ? p.qa.sn : p.qb.sn, row0, p.N, lane);
+            wait_tile_loads();  // settle the reload here so that later waits never have to cover it
             q_held = which;
         }
     };
@@ -185,23 +186,21 @@ __global__ __launch_bounds__(kThreads, 2) void window_kernel(Params p) {
         v_copy.load(s_v[0], v_src, p.v.sn, u_lo * kBN, p.N);
     }
 
-    auto prefetch = [&](int n0_next, int into) {  // K of the tile's main pair + V, into buffer `into`
-        const int src = classify<MODE>(rules, m0, m1, n0_next).main;
-        k_copy.load(s_k[into], k_ptr(src), k_stride(src), n0_next, p.N);
-        v_copy.load(s_v[into], v_src, p.v.sn, n0_next, p.N);
-    };
-
-    for (int u = u_lo; u < u_hi; ++u) {
+    // One key tile: operands from the current buffers while the next tile streams into the other pair.
+    auto tile_step = [&](const char* cur_k, const char* cur_v, char* nxt_k, char* nxt_v, int u) {
         const int n0 = u * kBN;
         const bool more = u + 1 < u_hi;
         const TileClass tc = classify<MODE>(rules, m0, m1, n0);
-        wait_tile_loads();
-        __syncthreads();  // tile u is complete in `buf`; every wave is done with the other buffer
+        auto prefetch = [&]() {  // K of the next tile's main pair + V, into the next buffers
+            const int src = classify<MODE>(rules, m0, m1, n0 + kBN).main;
+            k_copy.load(nxt_k, k_ptr(src), k_stride(src), n0 + kBN, p.N);
+            v_copy.load(nxt_v, v_src, p.v.sn, n0 + kBN, p.N);
+        };
         hold_q(kDual && tc.main != 0 ? 1 : 0);
-        if (tc.fast && more) prefetch(n0 + kBN, buf ^ 1);  // next tile's loads fly while this one is computed
+        if (tc.fast && more) prefetch();  // next tile's loads fly while this one is computed
 
         f32x16_t s[2];
-        qk_mma<Tag, D>(s, q, s_k[buf], lane);
+        qk_mma<Tag, D>(s, q, cur_k, lane);
         if (!tc.fast) {
             // tile on the diagonal / window edge / far-context boundary: every pair it touches, per-element
             // selection and masking
@@ -210,12 +209,12 @@ __global__ __launch_bounds__(kThreads, 2) void window_kernel(Params p) {
                 // the other pairs, one K tile at a time through the (still free) K buffer of the next tile
                 for (int src = 0; src < 3; ++src) {
                     if (src == tc.main || !((tc.need >> src) & 1)) continue;
-                    k_copy.load(s_k[buf ^ 1], k_ptr(src), k_stride(src), n0, p.N);
+                    k_copy.load(nxt_k, k_ptr(src), k_stride(src), n0, p.N);
                     hold_q(src == 0 ? 0 : 1);
                     wait_tile_loads();
                     __syncthreads();
                     f32x16_t s2[2];
-                    qk_mma<Tag, D>(s2, q, s_k[buf ^ 1], lane);
+                    qk_mma<Tag, D>(s2, q, nxt_k, lane);
 #pragma unroll
                     for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
@@ -233,12 +232,18 @@ __global__ __launch_bounds__(kThreads, 2) void window_kernel(Params p) {
                     const int j = n0 + kb * 32 + key_of_reg(r, half);
                     s[kb][r] = rules.visible(qi, j) ? s[kb][r] : -INFINITY;
                 }
-            if (more) prefetch(n0 + kBN, buf ^ 1);
+            if (more) prefetch();
         }
 
         vec8 pf[2][2];
         softmax_update<Tag, D, false>(st, s, p.scale_log2e, pf, nullptr);
-        pv_mma<Tag, D>(st.o, pf, s_v[buf], lane);
+        pv_mma<Tag, D>(st.o, pf, cur_v, lane);
+    };
+
+    for (int u = u_lo; u < u_hi; ++u) {
+        wait_tile_loads();
+        __syncthreads();  // tile u is complete in `buf`; every wave is done with the other buffer
+        tile_step(s_k[buf], s_v[buf], s_k[buf ^ 1], s_v[buf ^ 1], u);
         buf ^= 1;
     }
 
