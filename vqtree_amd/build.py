@@ -16,6 +16,7 @@ HIPCC_FLAGS = [
     "-shared",
     "-Wall",
     "-Wno-unused-function",
+    "-Wno-inline-asm",
     # packed fp32 VALU ops stay off for device code
     "-Xclang",
     "-target-feature",

@@ -17,6 +17,16 @@
 
 #include "vqa_common.h"
 
+// wave priority while a wave issues its MFMA bursts (0 = leave the default)
+#ifndef VQA_MFMA_PRIO_LEVEL
+#define VQA_MFMA_PRIO_LEVEL 0
+#endif
+#if VQA_MFMA_PRIO_LEVEL > 0
+#define VQA_MFMA_PRIO(on) __builtin_amdgcn_s_setprio((on) ? VQA_MFMA_PRIO_LEVEL : 0)
+#else
+#define VQA_MFMA_PRIO(on) ((void)0)
+#endif
+
 namespace vqa {
 namespace flash {
 
@@ -119,17 +129,21 @@ struct TileCopy {
     __device__ __forceinline__ uint32_t dst(const char* lds_tile, int i) const {
         return lds_addr_of(lds_tile) + (wave * Geom<D>::kRowsPerWave + i * Geom<D>::kRowsPerInstr) * Geom<D>::kRowBytes;
     }
-    // rows [n0, n0+64) of a [n_rows, D] matrix with row stride sn (elements); rows past the end repeat the last row
-    __device__ __forceinline__ void load(char* lds_tile, const uint16_t* base, int64_t sn, int n0, int n_rows) const {
-        if (n0 + kBN <= n_rows) {
-            // uniform (scalar) tile/row-group base + one 32-bit per-lane offset
-            const uint32_t lane_off = (uint32_t)lane_row * (uint32_t)(sn * 2);
+    // rows [n0, n0+64), all inside the matrix: uniform (scalar) row-group base + one 32-bit per-lane offset
+    __device__ __forceinline__ void load_full(const char* lds_tile, const uint16_t* base, int64_t sn, int n0) const {
+        const uint32_t lane_off = (uint32_t)lane_row * (uint32_t)(sn * 2);
 #pragma unroll
-            for (int i = 0; i < Geom<D>::kInstr; ++i) {
-                const char* grp = reinterpret_cast<const char*>(
-                    base + (int64_t)(n0 + wave * Geom<D>::kRowsPerWave + i * Geom<D>::kRowsPerInstr) * sn);
-                dma16(grp + (lane_off + chunk_bytes[i]), dst(lds_tile, i));
-            }
+        for (int i = 0; i < Geom<D>::kInstr; ++i) {
+            const char* grp = reinterpret_cast<const char*>(
+                base + (int64_t)(n0 + wave * Geom<D>::kRowsPerWave + i * Geom<D>::kRowsPerInstr) * sn);
+            dma16(grp + (lane_off + chunk_bytes[i]), dst(lds_tile, i));
+        }
+    }
+    // rows [n0, n0+64) of a [n_rows, D] matrix with row stride sn (elements); rows past the end repeat the last row
+    __device__ __forceinline__ void load(const char* lds_tile, const uint16_t* base, int64_t sn, int n0,
+                                         int n_rows) const {
+        if (n0 + kBN <= n_rows) {
+            load_full(lds_tile, base, sn, n0);
         } else {
 #pragma unroll
             for (int i = 0; i < Geom<D>::kInstr; ++i) {
@@ -140,7 +154,7 @@ struct TileCopy {
         }
     }
     // same with the global row taken from an index list
-    __device__ __forceinline__ void load_gather(char* lds_tile, const uint16_t* base, int64_t sn,
+    __device__ __forceinline__ void load_gather(const char* lds_tile, const uint16_t* base, int64_t sn,
                                                 const int64_t* row_index, int n0, int n_rows) const {
 #pragma unroll
         for (int i = 0; i < Geom<D>::kInstr; ++i) {
@@ -173,25 +187,27 @@ __device__ __forceinline__ void qk_mma(f32x16_t (&s)[2], const QFrag<Tag, D>& q,
     typedef const __attribute__((address_space(3))) vec8* lds_vec8_ptr;
     const uint32_t base = (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) char*)lds_k +
                           ((uint32_t)(r * G::kRowBytes) | (uint32_t)((half ^ G::swz_k(r)) << 4));
+    // step n works on key block n % 2 and k-step n / 2: the two accumulation chains alternate, so an MFMA never
+    // has to wait for the one issued just before it
     auto frag = [&](int n) {
-        const uint32_t addr = (base ^ (uint32_t)((2 * (n % KS)) << 4)) + (n / KS) * 32 * G::kRowBytes;
+        const uint32_t addr = (base ^ (uint32_t)((2 * (n / 2)) << 4)) + (n % 2) * 32 * G::kRowBytes;
         return *(lds_vec8_ptr)(uintptr_t)addr;
     };
     vec8 a[kAhead + 1];
 #pragma unroll
     for (int i = 0; i < kAhead; ++i) a[i] = frag(i);
-    f32x16_t acc;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) s[kb][e] = 0.f;
+    VQA_MFMA_PRIO(1);
 #pragma unroll
     for (int i = 0; i < kSteps; ++i) {
         if (i + kAhead < kSteps) a[(i + kAhead) % (kAhead + 1)] = frag(i + kAhead);
-        if (i % KS == 0) {
-#pragma unroll
-            for (int e = 0; e < 16; ++e) acc[e] = 0.f;
-        }
-        acc = Elem<Tag>::mfma32(a[i % (kAhead + 1)], q.f[i % KS], acc);
-        if (i % KS == KS - 1) s[i / KS] = acc;
+        s[i % 2] = Elem<Tag>::mfma32(a[i % (kAhead + 1)], q.f[i / 2], s[i % 2]);
         __builtin_amdgcn_sched_barrier(0);
     }
+    VQA_MFMA_PRIO(0);
 }
 
 // key offset inside a 32-key block held at accumulator register r by a lane of the given half
@@ -229,6 +245,7 @@ __device__ __forceinline__ void pv_mma(f32x16_t (&o)[Geom<D>::kDBlocks], const t
     };
 #pragma unroll
     for (int i = 0; i < kAhead; ++i) fetch(i);
+    VQA_MFMA_PRIO(1);
 #pragma unroll
     for (int i = 0; i < kSteps; ++i) {
         if (i + kAhead < kSteps) fetch(i + kAhead);
@@ -238,6 +255,7 @@ __device__ __forceinline__ void pv_mma(f32x16_t (&o)[Geom<D>::kDBlocks], const t
         o[i % DB] = Elem<Tag>::mfma32(__builtin_bit_cast(vec8, av), p[kbj >> 1][kbj & 1], o[i % DB]);
         __builtin_amdgcn_sched_barrier(0);
     }
+    VQA_MFMA_PRIO(0);
 }
 
 // Online-softmax state of one wave: every lane carries the running max of ITS query (identical in lane ^ 32) and

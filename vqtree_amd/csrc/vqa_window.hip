@@ -33,6 +33,7 @@ struct Params {
     int causal;
     int boundary;  // Boundary, kVqPrefill only
     int has_b;     // kVqPrefill: pair B is distinct from pair A (q2 and k2 both given)
+    int pair_tiles;  // a workgroup handles query tiles (n-1-k, k) instead of one tile
     float scale_log2e;
 };
 
@@ -125,23 +126,25 @@ __global__ __launch_bounds__(kThreads, 2) void window_kernel(Params p) {
     const int half = lane >> 5, nq = lane & 31;
     // Workgroups are dispatched round-robin over the 8 XCDs (each with its own L2) in linear-id order.  Give every
     // XCD whole (batch, head) problems: the query tiles of one head then share its K/V through one L2.
-    int bh, t;
+    // With `pair_tiles` a workgroup takes query tile k from the end AND tile k from the start, so that under a
+    // causal mask every workgroup does the same amount of work.
+    const int n_tiles = (p.N + kBM - 1) / kBM;
+    int bh, slot;
     {
-        const int n_tiles = gridDim.x, n_bh = gridDim.y;
-        const int id = blockIdx.x + n_tiles * blockIdx.y;
+        const int n_slots = gridDim.x, n_bh = gridDim.y;
+        const int id = blockIdx.x + n_slots * blockIdx.y;
         if (n_bh % 8 == 0) {
             const int xcd = id & 7, k = id >> 3;
-            bh = xcd + 8 * (k / n_tiles);
-            t = n_tiles - 1 - (k % n_tiles);  // long (late) query tiles first
+            bh = xcd + 8 * (k / n_slots);
+            slot = k % n_slots;
         } else {
             bh = blockIdx.y;
-            t = n_tiles - 1 - blockIdx.x;
+            slot = blockIdx.x;
         }
     }
     const int b = bh / p.H, h = bh % p.H;
-    const int m0 = t * kBM;
-    const int m1 = min(m0 + kBM - 1, p.N - 1);
-    const int row0 = m0 + wave * 32;
+    const int t_first = n_tiles - 1 - slot;  // long (late) query tiles are scheduled first
+    const int n_pass = (p.pair_tiles && slot != t_first) ? 2 : 1;
 
     Rules<MODE> rules{p.N, p.window, p.causal, p.boundary, p.has_b};
 
@@ -151,6 +154,18 @@ __global__ __launch_bounds__(kThreads, 2) void window_kernel(Params p) {
     const uint16_t* v_src = p.v.p + b * p.v.sb + h * p.v.sh;
     auto k_ptr = [&](int src) { return src == 0 ? ka : (src == 1 ? kb_ : kc); };
     auto k_stride = [&](int src) { return src == 0 ? p.ka.sn : (src == 1 ? p.kb.sn : p.kc.sn); };
+
+    TileCopy<D, false> k_copy;
+    TileCopy<D, true> v_copy;
+    k_copy.init(wave, lane);
+    v_copy.init(wave, lane);
+
+    for (int pass = 0; pass < n_pass; ++pass) {
+    const int t = pass == 0 ? t_first : slot;
+    const int m0 = t * kBM;
+    const int m1 = min(m0 + kBM - 1, p.N - 1);
+    const int row0 = m0 + wave * 32;
+    if (pass) __syncthreads();  // the previous tile's last reads of the LDS buffers are done
 
     // One query fragment set lives in registers: pair A's or pair B's.  Tiles are visited far -> near, so the
     // operand in use changes O(1) times per workgroup; a change re-reads the wave's 32 rows (L2 hits).
@@ -165,11 +180,6 @@ __global__ __launch_bounds__(kThreads, 2) void window_kernel(Params p) {
             q_held = which;
         }
     };
-
-    TileCopy<D, false> k_copy;
-    TileCopy<D, true> v_copy;
-    k_copy.init(wave, lane);
-    v_copy.init(wave, lane);
 
     // key tiles this workgroup visits
     const int hi_key = rules.is_causal() ? min(p.N, m1 + 1) : p.N;
@@ -186,45 +196,76 @@ __global__ __launch_bounds__(kThreads, 2) void window_kernel(Params p) {
         v_copy.load(s_v[0], v_src, p.v.sn, u_lo * kBN, p.N);
     }
 
-    // One key tile: operands from the current buffers while the next tile streams into the other pair.
-    auto tile_step = [&](const char* cur_k, const char* cur_v, char* nxt_k, char* nxt_v, int u) {
-        const int n0 = u * kBN;
-        const bool more = u + 1 < u_hi;
-        const TileClass tc = classify<MODE>(rules, m0, m1, n0);
-        auto prefetch = [&]() {  // K of the next tile's main pair + V, into the next buffers
-            const int src = classify<MODE>(rules, m0, m1, n0 + kBN).main;
-            k_copy.load(nxt_k, k_ptr(src), k_stride(src), n0 + kBN, p.N);
-            v_copy.load(nxt_v, v_src, p.v.sn, n0 + kBN, p.N);
-        };
-        hold_q(kDual && tc.main != 0 ? 1 : 0);
-        if (tc.fast && more) prefetch();  // next tile's loads fly while this one is computed
+    // scores -> probabilities -> O update for the tile whose K / V sit in cur_k / cur_v
+    auto attend_tile = [&](f32x16_t(&s)[2], const char* cur_v) {
+        vec8 pf[2][2];
+        softmax_update<Tag, D, false>(st, s, p.scale_log2e, pf, nullptr);
+        pv_mma<Tag, D>(st.o, pf, cur_v, lane);
+    };
 
-        f32x16_t s[2];
-        qk_mma<Tag, D>(s, q, cur_k, lane);
-        if (!tc.fast) {
-            // tile on the diagonal / window edge / far-context boundary: every pair it touches, per-element
-            // selection and masking
-            const int qi = row0 + nq;
-            if constexpr (kDual) {
-                // the other pairs, one K tile at a time through the (still free) K buffer of the next tile
-                for (int src = 0; src < 3; ++src) {
-                    if (src == tc.main || !((tc.need >> src) & 1)) continue;
-                    k_copy.load(nxt_k, k_ptr(src), k_stride(src), n0, p.N);
-                    hold_q(src == 0 ? 0 : 1);
-                    wait_tile_loads();
-                    __syncthreads();
-                    f32x16_t s2[2];
-                    qk_mma<Tag, D>(s2, q, nxt_k, lane);
-#pragma unroll
-                    for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                        for (int r = 0; r < 16; ++r) {
-                            const int j = n0 + kb * 32 + key_of_reg(r, half);
-                            if (rules.source(qi, j) == src) s[kb][r] = s2[kb][r];
-                        }
-                    __syncthreads();  // all waves have read this pair's K tile before the buffer is reused
-                }
+    int u = u_lo;
+    while (u < u_hi) {
+        const TileClass tc = classify<MODE>(rules, m0, m1, u * kBN);
+        // length of the run of tiles that use this same single pair with no mask (whole tiles, in range)
+        int u_end = u;
+        if (tc.fast) {
+            u_end = u + 1;
+            while (u_end < u_hi) {
+                const TileClass t2 = classify<MODE>(rules, m0, m1, u_end * kBN);
+                if (!t2.fast || t2.main != tc.main) break;
+                ++u_end;
             }
+        }
+        if (u_end - u >= 2) {
+            // hot loop: tiles u .. u_end-2 (the run's last tile goes through the general path below, which also
+            // knows how to fetch whatever follows the run)
+            hold_q(kDual && tc.main != 0 ? 1 : 0);
+            const uint16_t* run_k = k_ptr(tc.main);
+            const int64_t run_sn = k_stride(tc.main);
+            for (; u < u_end - 1; ++u) {
+                wait_tile_loads();
+                __syncthreads();  // tile u is complete in `buf`; every wave is done with the other buffer
+                k_copy.load_full(s_k[buf ^ 1], run_k, run_sn, (u + 1) * kBN);
+                v_copy.load_full(s_v[buf ^ 1], v_src, p.v.sn, (u + 1) * kBN);
+                f32x16_t s[2];
+                qk_mma<Tag, D>(s, q, s_k[buf], lane);
+                attend_tile(s, s_v[buf]);
+                buf ^= 1;
+            }
+        }
+
+        // general tile: every pair it touches, per-element selection and masking
+        const int n0 = u * kBN;
+        const TileClass tg = classify<MODE>(rules, m0, m1, n0);
+        const char* cur_k = s_k[buf];
+        const char* nxt_k = s_k[buf ^ 1];
+        wait_tile_loads();
+        __syncthreads();
+        const int qi = row0 + nq;
+        f32x16_t s[2];
+        hold_q(kDual && tg.main != 0 ? 1 : 0);
+        qk_mma<Tag, D>(s, q, cur_k, lane);
+        if constexpr (kDual) {
+            // the other pairs, one K tile at a time through the (still free) K buffer of the next tile
+            for (int src = 0; src < 3; ++src) {
+                if (src == tg.main || !((tg.need >> src) & 1)) continue;
+                k_copy.load(nxt_k, k_ptr(src), k_stride(src), n0, p.N);
+                hold_q(src == 0 ? 0 : 1);
+                wait_tile_loads();
+                __syncthreads();
+                f32x16_t s2[2];
+                qk_mma<Tag, D>(s2, q, nxt_k, lane);
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int j = n0 + kb * 32 + key_of_reg(r, half);
+                        if (rules.source(qi, j) == src) s[kb][r] = s2[kb][r];
+                    }
+                __syncthreads();  // all waves have read this pair's K tile before the buffer is reused
+            }
+        }
+        if (!tg.fast) {
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
@@ -232,28 +273,29 @@ __global__ __launch_bounds__(kThreads, 2) void window_kernel(Params p) {
                     const int j = n0 + kb * 32 + key_of_reg(r, half);
                     s[kb][r] = rules.visible(qi, j) ? s[kb][r] : -INFINITY;
                 }
-            if (more) prefetch();
         }
-
-        vec8 pf[2][2];
-        softmax_update<Tag, D, false>(st, s, p.scale_log2e, pf, nullptr);
-        pv_mma<Tag, D>(st.o, pf, cur_v, lane);
-    };
-
-    for (int u = u_lo; u < u_hi; ++u) {
-        wait_tile_loads();
-        __syncthreads();  // tile u is complete in `buf`; every wave is done with the other buffer
-        tile_step(s_k[buf], s_v[buf], s_k[buf ^ 1], s_v[buf ^ 1], u);
+        if (u + 1 < u_hi) {
+            const int src = classify<MODE>(rules, m0, m1, n0 + kBN).main;
+            k_copy.load(nxt_k, k_ptr(src), k_stride(src), n0 + kBN, p.N);
+            v_copy.load(s_v[buf ^ 1], v_src, p.v.sn, n0 + kBN, p.N);
+        }
+        attend_tile(s, s_v[buf]);
         buf ^= 1;
+        ++u;
     }
 
     store_output<Tag, D>(st, p.out + b * p.o_sb + h * p.o_sh, p.o_sn,
                          p.lse ? p.lse + (int64_t)bh * p.N : nullptr, row0, p.N, lane);
+    }
 }
 
 template <typename Tag, int D, int MODE>
-int launch(const Params& p, int B, hipStream_t stream) {
-    const dim3 grid((p.N + kBM - 1) / kBM, B * p.H);
+int launch(Params p, int B, hipStream_t stream) {
+    const int n_tiles = (p.N + kBM - 1) / kBM;
+    // Pair late (long) and early (short) query tiles whenever enough workgroups remain to fill the 256 CUs twice
+    // over: under a causal mask every workgroup then does the same amount of work.
+    p.pair_tiles = ((int64_t)(n_tiles / 2) * B * p.H >= 1024) ? 1 : 0;
+    const dim3 grid(p.pair_tiles ? (n_tiles + 1) / 2 : n_tiles, B * p.H);
     hipLaunchKernelGGL((window_kernel<Tag, D, MODE>), grid, dim3(kThreads), 0, stream, p);
     return launch_status();
 }
