@@ -60,12 +60,67 @@ def cpu_baseline(case, units=32, repeats=3):
     }
 
 
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
+
+
+def _time_events(fn, steps, warmup):
+    import torch
+
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    for i in range(steps):
+        starts[i].record()
+        fn()
+        ends[i].record()
+    torch.cuda.synchronize()
+    ms = sorted(s.elapsed_time(e) for s, e in zip(starts, ends))
+    return ms[len(ms) // 2]
+
+
+def prefill_extra(dev, steps=20, warmup=5):
+    """Second half of the metric: causal VQ-attention prefill at 8k with a 1024-key exact window (not part of the
+    timed decode region).  Reported as algorithmic TFLOP/s and as a fraction of the bf16 MFMA peak."""
+    import torch
+
+    from vqtree_amd.ops.attn_vq import attn_vq_prefill
+    from vqtree_amd.synthetic import prefill_c3
+
+    case = prefill_c3(dev)
+    fn = lambda: attn_vq_prefill(case.q, case.codes, case.codebooks, case.v, k_exact=case.k_exact,
+                                 window_size=case.window, softmax_scale=case.softmax_scale)
+    ms = _time_events(fn, steps, warmup)
+    flops = case.algorithmic_flops("block")
+    B, H, N, D = case.q.shape
+    tf = flops / (ms * 1e-3) / 1e12
+    out = {
+        "workload": f"causal VQ-attention prefill: batch {B}, {H} heads, head_dim {D}, seq {N}, exact window "
+                    f"{case.window} (block boundary rule), {case.codes.shape[3]} codebooks x "
+                    f"{case.codebooks.shape[2]}, bf16",
+        "us_per_call": round(ms * 1e3, 1),
+        "algorithmic_gflop": round(flops / 1e9, 2),
+        "tflops": round(tf, 1),
+        "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
+                     "duration_covers": "whole call: key reconstruction kernel + fused window/far attention kernel"},
+    }
+    del case
+    torch.cuda.empty_cache()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-prefill", action="store_true", help="skip the (untimed-region) prefill measurement")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="before the timed region, run one plain 1 GiB device copy (reference dispatch of known "
+                         "size for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU only: the VQ-attention path shards over (batch, head) with no "
@@ -88,6 +143,13 @@ def main():
     def step():
         return attn_vq_decode(case.q, case.codes, case.codebooks, case.v, softmax_scale=case.softmax_scale)
 
+    if args.calibrate_copy:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)  # reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -143,6 +205,10 @@ def main():
     }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(case)
+    if not args.no_prefill:
+        del case
+        torch.cuda.empty_cache()
+        result["prefill"] = prefill_extra(dev)
     print(json.dumps(result))
 
 

@@ -210,6 +210,28 @@ __device__ __forceinline__ void qk_mma(f32x16_t (&s)[2], const QFrag<Tag, D>& q,
     VQA_MFMA_PRIO(0);
 }
 
+// One 32-key block of S^T (key block kb of the tile), for the rarely taken multi-pair tiles where register
+// pressure matters more than pipelining.
+template <typename Tag, int D>
+__device__ __forceinline__ f32x16_t qk_block(const QFrag<Tag, D>& q, const char* lds_k, int kb, int lane) {
+    typedef typename Elem<Tag>::vec8 vec8;
+    typedef Geom<D> G;
+    typedef const __attribute__((address_space(3))) vec8* lds_vec8_ptr;
+    const int r = lane & 31, half = lane >> 5;
+    const uint32_t base = lds_addr_of(lds_k) + kb * 32 * G::kRowBytes +
+                          ((uint32_t)(r * G::kRowBytes) | (uint32_t)((half ^ G::swz_k(r)) << 4));
+    f32x16_t acc;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[e] = 0.f;
+#pragma unroll
+    for (int kk = 0; kk < G::kKSteps; ++kk) {
+        const vec8 a = *(lds_vec8_ptr)(uintptr_t)(base ^ (uint32_t)((2 * kk) << 4));
+        acc = Elem<Tag>::mfma32(a, q.f[kk], acc);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    return acc;
+}
+
 // key offset inside a 32-key block held at accumulator register r by a lane of the given half
 __device__ __forceinline__ int key_of_reg(int r, int half) { return 8 * (r >> 2) + 4 * half + (r & 3); }
 

@@ -18,7 +18,8 @@ enum Mode : int {
     kLocalLoose = 1,   // j <= i, j >= floor(i/T)*T - W                           (one pair)
     kLocalRerope = 2,  // visible as loose; pair A iff i - j <= W, else pair B
     kFullRerope = 3,   // all keys (causal optional); pair A iff |i - j| < W, else pair B
-    kVqPrefill = 4     // causal optional; j < far_bnd(i) -> pair C; else A iff i - j <= W, else B
+    kVqPrefill = 4,    // causal optional; j < far_bnd(i) -> pair C; else A iff i - j <= W, else B
+    kVqPrefill2 = 5    // same without a distinct pair B (no q2/k2 strip): two pairs, lower register pressure
 };
 
 enum Boundary : int { kBoundaryBlock = 0, kBoundaryExact = 1, kBoundaryAllFar = 2 };
@@ -55,19 +56,21 @@ struct Rules {
         if (MODE == kLocalLoose || MODE == kLocalRerope) return (i / kTile) * kTile - W;
         return 0;
     }
-    __device__ __forceinline__ bool is_causal() const {
-        return (MODE == kFullRerope || MODE == kVqPrefill) ? causal != 0 : true;
-    }
-    __device__ __forceinline__ bool visible(int i, int j) const {
-        return j < N && (!is_causal() || j <= i) && j >= vis_lo(i);
+    static constexpr bool kIsVq = (MODE == kVqPrefill || MODE == kVqPrefill2);
+    __device__ __forceinline__ bool pair_b() const { return MODE == kVqPrefill2 ? false : has_b != 0; }
+    __device__ __forceinline__ bool is_causal() const { return (MODE == kFullRerope || kIsVq) ? causal != 0 : true; }
+    // Per-element predicates take the row's bounds precomputed (they depend on the query only):
+    // lo = vis_lo(i), fb = far_bnd(i).
+    __device__ __forceinline__ bool visible(int i, int j, int lo) const {
+        return j < N && (!is_causal() || j <= i) && j >= lo;
     }
     // 0 = A, 1 = B, 2 = C
-    __device__ __forceinline__ int source(int i, int j) const {
+    __device__ __forceinline__ int source(int i, int j, int fb) const {
         if (MODE == kLocalStrict || MODE == kLocalLoose) return 0;
         if (MODE == kLocalRerope) return (i - j <= W) ? 0 : 1;
         if (MODE == kFullRerope) return (abs(i - j) < W) ? 0 : 1;
-        if (j < far_bnd(i)) return 2;
-        return (i - j <= W || !has_b) ? 0 : 1;
+        if (j < fb) return 2;
+        return (i - j <= W || !pair_b()) ? 0 : 1;
     }
 };
 
@@ -96,11 +99,11 @@ __device__ __forceinline__ TileClass classify(const Rules<MODE>& r, int m0, int 
         allA = dmax < r.W && dmin > -r.W;
         needB = !allA;
         allB = !needA;
-    } else if (MODE == kVqPrefill) {
+    } else if (Rules<MODE>::kIsVq) {
         needC = n0 < r.far_bnd(m1);
         allC = n1 < r.far_bnd(m0);
-        needB = !allC && r.has_b && dmax > r.W;
-        needA = !allC && (dmin <= r.W || !r.has_b);
+        needB = !allC && r.pair_b() && dmax > r.W;
+        needA = !allC && (dmin <= r.W || !r.pair_b());
         allA = !needC && !needB;
         allB = !needC && !needA;
     }
@@ -114,7 +117,7 @@ template <typename Tag, int D, int MODE>
 __global__ __launch_bounds__(kThreads, 2) void window_kernel(Params p) {
     typedef Geom<D> G;
     typedef typename Elem<Tag>::vec8 vec8;
-    constexpr bool kDual = (MODE == kLocalRerope || MODE == kFullRerope || MODE == kVqPrefill);
+    constexpr bool kDual = (MODE == kLocalRerope || MODE == kFullRerope || MODE == kVqPrefill || MODE == kVqPrefill2);
 
     // double-buffered K and V tiles, filled by direct global -> LDS loads one tile ahead of the compute
     __shared__ __attribute__((aligned(1024))) char s_k[2][G::kTileBytes];
@@ -165,6 +168,9 @@ __global__ __launch_bounds__(kThreads, 2) void window_kernel(Params p) {
     const int m0 = t * kBM;
     const int m1 = min(m0 + kBM - 1, p.N - 1);
     const int row0 = m0 + wave * 32;
+    const int qi = row0 + nq;  // this lane's query and its row bounds
+    const int qi_vis_lo = rules.vis_lo(qi);
+    const int qi_far_bnd = Rules<MODE>::kIsVq ? rules.far_bnd(qi) : 0;
     if (pass) __syncthreads();  // the previous tile's last reads of the LDS buffers are done
 
     // One query fragment set lives in registers: pair A's or pair B's.  Tiles are visited far -> near, so the
@@ -241,27 +247,28 @@ __global__ __launch_bounds__(kThreads, 2) void window_kernel(Params p) {
         const char* nxt_k = s_k[buf ^ 1];
         wait_tile_loads();
         __syncthreads();
-        const int qi = row0 + nq;
         f32x16_t s[2];
         hold_q(kDual && tg.main != 0 ? 1 : 0);
         qk_mma<Tag, D>(s, q, cur_k, lane);
         if constexpr (kDual) {
             // the other pairs, one K tile at a time through the (still free) K buffer of the next tile
             for (int src = 0; src < 3; ++src) {
+                if (MODE == kVqPrefill2 && src == 1) continue;
+                if (MODE != kVqPrefill && MODE != kVqPrefill2 && src == 2) continue;
                 if (src == tg.main || !((tg.need >> src) & 1)) continue;
                 k_copy.load(nxt_k, k_ptr(src), k_stride(src), n0, p.N);
                 hold_q(src == 0 ? 0 : 1);
                 wait_tile_loads();
                 __syncthreads();
-                f32x16_t s2[2];
-                qk_mma<Tag, D>(s2, q, nxt_k, lane);
 #pragma unroll
-                for (int kb = 0; kb < 2; ++kb)
+                for (int kb = 0; kb < 2; ++kb) {
+                    const f32x16_t s2 = qk_block<Tag, D>(q, nxt_k, kb, lane);
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
                         const int j = n0 + kb * 32 + key_of_reg(r, half);
-                        if (rules.source(qi, j) == src) s[kb][r] = s2[kb][r];
+                        if (rules.source(qi, j, qi_far_bnd) == src) s[kb][r] = s2[r];
                     }
+                }
                 __syncthreads();  // all waves have read this pair's K tile before the buffer is reused
             }
         }
@@ -271,7 +278,7 @@ __global__ __launch_bounds__(kThreads, 2) void window_kernel(Params p) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int j = n0 + kb * 32 + key_of_reg(r, half);
-                    s[kb][r] = rules.visible(qi, j) ? s[kb][r] : -INFINITY;
+                    s[kb][r] = rules.visible(qi, j, qi_vis_lo) ? s[kb][r] : -INFINITY;
                 }
         }
         if (u + 1 < u_hi) {
@@ -307,7 +314,8 @@ int dispatch_mode(const Params& p, int B, int mode, hipStream_t stream) {
         case kLocalLoose: return launch<Tag, D, kLocalLoose>(p, B, stream);
         case kLocalRerope: return launch<Tag, D, kLocalRerope>(p, B, stream);
         case kFullRerope: return launch<Tag, D, kFullRerope>(p, B, stream);
-        case kVqPrefill: return launch<Tag, D, kVqPrefill>(p, B, stream);
+        case kVqPrefill:
+            return p.has_b ? launch<Tag, D, kVqPrefill>(p, B, stream) : launch<Tag, D, kVqPrefill2>(p, B, stream);
         default: return VQA_ERR_BAD_ARGUMENT;
     }
 }

@@ -52,3 +52,52 @@ def decode_case(B, H, N, D, M, K=256, dtype=torch.bfloat16, device="cuda", seed=
 def decode_c2(device="cuda"):
     """Decode benchmark: batch 16, 32 heads, head_dim 128, 32768 keys, 4 codebooks x 256 codewords, bf16."""
     return decode_case(16, 32, 32768, 128, 4, 256, torch.bfloat16, device, seed=2, cb_std=0.35, on_device=True)
+
+
+@dataclass
+class PrefillCase:
+    q: torch.Tensor          # [B,H,N,D]
+    k_exact: torch.Tensor    # [B,H,N,D] exact keys of the sliding window
+    v: torch.Tensor          # [B,H,N,D]
+    codes: torch.Tensor      # [B,H,N,M] uint8
+    codebooks: torch.Tensor  # [H,M,K,D]
+    window: int
+    softmax_scale: float
+
+    def algorithmic_flops(self, boundary_mode="block") -> int:
+        """LUT (2*N*M*K*D) + exact QK^T (2*D*P_exact) + P.V (2*D*(P_exact + P_far)) per (batch, head), pairs counted
+        from the mask: P_far = sum_i boundary(i), P_exact = sum_i (i + 1 - boundary(i))."""
+        B, H, N, D = self.q.shape
+        M, K = self.codes.shape[3], self.codebooks.shape[2]
+        i = torch.arange(N, dtype=torch.int64)
+        if boundary_mode == "block":
+            bnd = torch.clamp(torch.div(i - self.window, 128, rounding_mode="floor") * 128, min=0)
+        else:
+            bnd = torch.clamp(i - self.window, min=0)
+        p_far = int(bnd.sum())
+        p_exact = int((i + 1 - bnd).sum())
+        per_head = 2 * N * M * K * D + 2 * D * p_exact + 2 * D * (p_exact + p_far)
+        return B * H * per_head
+
+
+def prefill_case(B, H, N, D, M, W, K=256, dtype=torch.bfloat16, device="cuda", seed=3, cb_std=0.35, on_device=False):
+    """q, k_exact, V ~ N(0,1); codebooks ~ N(0, cb_std); codes uniform in [0,K)."""
+    if on_device:
+        g = torch.Generator(device=device).manual_seed(seed)
+        mk = lambda *s: torch.randn(*s, generator=g, device=device, dtype=torch.float32)
+        q, k, v = mk(B, H, N, D).to(dtype), mk(B, H, N, D).to(dtype), mk(B, H, N, D).to(dtype)
+        cb = (mk(H, M, K, D) * cb_std).to(dtype)
+        codes = torch.randint(0, K, (B, H, N, M), generator=g, device=device, dtype=torch.uint8)
+    else:
+        g = torch.Generator("cpu").manual_seed(seed)
+        mk = lambda *s: torch.randn(*s, generator=g)
+        q, k, v = (mk(B, H, N, D).to(dtype).to(device) for _ in range(3))
+        cb = (mk(H, M, K, D) * cb_std).to(dtype).to(device)
+        codes = torch.randint(0, K, (B, H, N, M), generator=g, dtype=torch.int32).to(torch.uint8).to(device)
+    return PrefillCase(q, k, v, codes, cb, W, 1.0 / math.sqrt(D))
+
+
+def prefill_c3(device="cuda"):
+    """Prefill benchmark, Llama-2-7B shape: batch 1, 32 heads, head_dim 128, 8192 tokens, exact window 1024,
+    4 codebooks x 256 codewords, bf16 (codebook std 0.35, not fixed by the configuration)."""
+    return prefill_case(1, 32, 8192, 128, 4, 1024, device=device, seed=3, on_device=True)
