@@ -18,6 +18,9 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
+# HBM bytes one launch of the streaming kernel moves, from rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by a known copy
+# (profiles/decode_main_kernel_c2_b16_h32_n32768.md); valid for the default workload only
+DECODE_MAIN_KERNEL_TRAFFIC_BYTES = 4_380_977_000
 
 
 def cpu_baseline(case, units=32, repeats=3):
@@ -196,7 +199,7 @@ def main():
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
-            "traffic": None,
+            "traffic": DECODE_MAIN_KERNEL_TRAFFIC_BYTES,
             "kernel": "vqa::decode::main_kernel<bf16,128,4>",
             "duration_us": round(kern_ms * 1e3, 1),
             "duration_covers": "HIP events around the whole call (lookup-table + streaming + merge kernels); the "
