@@ -1,0 +1,90 @@
+"""GPU tests of the caller layer (the attention core of the reference's HF module): dispatch, preprocessing, the
+linear-time prefill against the per-query slow reference, and a generation step over the cached codes."""
+import math
+
+import pytest
+import torch
+
+import oracle
+from tests.util import assert_close_16
+from vqtree_amd.ops import attn_vq as A
+
+pytestmark = pytest.mark.gpu
+
+
+def _states(B, H, N, D, dtype, seed):
+    g = torch.Generator("cpu").manual_seed(seed)
+    mk = lambda: torch.randn(B, H, N, D, generator=g).to(dtype).cuda()
+    return mk(), mk(), mk()
+
+
+def test_reference_selfcheck_linear_vs_slow():
+    """The reference's own check (ops/attn_vq.py:534-556): 2 heads of dim 64, fp16, LEN = 511, window 256,
+    codebook randn(2,128,64); SORT_BASED_LINEAR against SLOW_REFERNECE through the dispatcher."""
+    print("callers: linear vs slow, LEN=511 W=256", flush=True)
+    B, H, N, D, W = 1, 2, 511, 64, 256
+    q, k, v = _states(B, H, N, D, torch.float16, 1)
+    codebook = torch.randn(H, 128, D, generator=torch.Generator("cpu").manual_seed(2)).half().cuda()
+    pos = torch.arange(N, device="cuda").unsqueeze(0)
+    fast = A.dispatch_attn(q, k, v, pos, A.VectorQuantizedReRoPECache(W, codebook))
+    slow = A.dispatch_attn(q, k, v, pos, A.VectorQuantizedReRoPECache(W, codebook, attention_mode=A.AttentionMode.SLOW_REFERNECE))
+    per_key = A.long_prefilling_per_key(q, k, v, pos, A.VectorQuantizedReRoPECache(W, codebook))
+    torch.cuda.synchronize()
+    assert fast.shape == (B, N, H * D)
+    assert (fast.float() - slow.float()).abs().max() <= 2e-2
+    assert (per_key.float() - slow.float()).abs().max() <= 2e-2
+    # rows inside the window see no far context: both fast paths are plain exact attention there
+    assert (fast[:, :W].float() - slow[:, :W].float()).abs().max() <= 1e-2
+
+
+def test_preprocess_matches_oracle_bit_exact_indices():
+    B, H, N, C, D = 2, 2, 640, 128, 64
+    _, k, v = _states(B, H, N, D, torch.bfloat16, 3)
+    cb = torch.randn(H, C, D, generator=torch.Generator("cpu").manual_seed(4)).to(torch.bfloat16).cuda()
+    _, ids, onehot = A.multi_head_single_quantize(k, cb)
+    cnt, v_vq, vi = A.sort_based_preprocess(ids, onehot, v)
+    want_cnt, want_vvq, want_vi = oracle.sort_based_preprocess(ids.cpu(), v.cpu(), C, dtype=torch.bfloat16)
+    assert torch.equal(cnt.cpu(), want_cnt) and torch.equal(vi.cpu(), want_vi)  # integer work: bit-exact
+    assert torch.allclose(v_vq.float().cpu(), want_vvq.float(), atol=3e-2, rtol=1e-2)  # fp32 cumsum order differs
+    # the encoder's ids are the first arg-max of the inner product evaluated in the model dtype
+    want_ids = oracle.multi_head_single_quantize(k.cpu(), cb.cpu())[1]
+    assert (ids.cpu() != want_ids).float().mean() < 5e-3  # bf16 matmul accumulation order may flip near-ties
+
+
+@pytest.mark.parametrize("N,W,C", [(900, 256, 256), (1536, 512, 128)])
+def test_linear_prefill_vs_oracle(N, W, C):
+    print(f"callers: linear prefill N{N} W{W} C{C}", flush=True)
+    B, H, D = 2, 2, 128
+    q, k, v = _states(B, H, N, D, torch.bfloat16, 5)
+    cb = torch.randn(H, C, D, generator=torch.Generator("cpu").manual_seed(6)).to(torch.bfloat16).cuda()
+    pos = torch.arange(N, device="cuda").unsqueeze(0).expand(B, -1)
+    cache = A.VectorQuantizedReRoPECache(W, cb)
+    out = A.dispatch_attn(q, k, v, pos, cache)
+    q1, k1, q2 = A.rerope_operands(q, k, pos, W)
+    ids = cache.key_codes[0]
+    want, _ = oracle.attn_vq_prefill(q1, ids, cb.unsqueeze(1), v, k_exact=k1, window_size=W, q2=q2, k2=k)
+    assert_close_16(out.view(B, N, H, D).transpose(1, 2), want, "linear prefill")
+
+
+def test_short_prefill_then_generation_steps():
+    """Prefill shorter than window + 128 is exact causal attention; each later seqlen_q == 1 step attends over the
+    cached key codes with the clamped query (dense oracle on the reconstructed keys)."""
+    B, H, N, D, W, C = 2, 4, 300, 128, 256, 256
+    q, k, v = _states(B, H, N, D, torch.bfloat16, 7)
+    cb = torch.randn(H, C, D, generator=torch.Generator("cpu").manual_seed(8)).to(torch.bfloat16).cuda()
+    pos = torch.arange(N, device="cuda").unsqueeze(0).expand(B, -1)
+    cache = A.VectorQuantizedReRoPECache(W, cb)
+    out = A.dispatch_attn(q, k, v, pos, cache)
+    q1, k1, _ = A.rerope_operands(q, k, pos, W)
+    want, _ = oracle.local_attn(q1, k1, v, N, "strict")
+    assert_close_16(out.view(B, N, H, D).transpose(1, 2), want, "short prefill")
+    assert cache.get_seq_length(0) == N and cache.seen_tokens == N
+    for step in range(3):
+        qs, ks, vs = _states(B, H, 1, D, torch.bfloat16, 20 + step)
+        o = A.dispatch_attn(qs, ks, vs, torch.full((B, 1), N + step, device="cuda"), cache)
+        n_now = N + step + 1
+        assert cache.get_seq_length(0) == n_now and o.shape == (B, 1, H * D)
+        cos, sin = A.rope_tables(D, W + 2, dtype=torch.bfloat16, device="cuda")
+        q2 = qs * cos[W + 1] + A.rotate_half(qs) * sin[W + 1]
+        want, _ = oracle.attn_vq_decode(q2, cache.key_codes[0], cb.unsqueeze(1), cache.value_cache[0], 1 / math.sqrt(D))
+        assert_close_16(o.view(B, 1, H, D).transpose(1, 2), want, f"generation step {step}")

@@ -5,10 +5,14 @@
 Layouts follow the reference's attention modules: q, v [B,H,N,D]; codebooks [H,M,K,D]; codes [B,H,N,M] uint8.
 """
 import math
+from enum import Enum
 
 import torch
 
 from .. import _lib
+from .mini_vq import multi_head_single_quantize
+
+BLOCK_SIZE = 128  # granularity of the far-context boundary (ops/attn_vq.py:23)
 
 _SUFFIX = {torch.bfloat16: "bf16", torch.float16: "f16"}
 
@@ -110,3 +114,187 @@ def attn_vq_prefill(q, k_codes, codebooks, v, *, k_exact=None, window_size=0, ca
             1 if causal else 0, softmax_scale, _lib.current_stream(q.device))
     _lib.check(rc)
     return (out, lse) if return_lse else out
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# Caller layer: the attention core of LlamaFlashAttention2VectorQuantizedReRoPE (ops/attn_vq.py:176-479) without the
+# Hugging Face module around it -- projections, o_proj and the transformers Cache base class stay with the model code.
+# ---------------------------------------------------------------------------------------------------------------------
+class AttentionMode(Enum):
+    SLOW_REFERNECE = 0  # (sic) spelling of the reference, ops/attn_vq.py:26-28
+    SORT_BASED_LINEAR = 1
+
+
+class VectorQuantizedReRoPECache:
+    """Holds what the reference's cache of the same name configures (ops/attn_vq.py:31-52): the exact-window length,
+    the per-head codebook [H,C,D], the `sphere` flag and the attention mode; plus, after a prefill, the decode state
+    (single-codebook key codes [B,H,N,1] uint8 when C <= 256, and V) so that seqlen_q == 1 steps can run
+    `attn_vq_decode`."""
+
+    def __init__(self, window_length, codebook, sphere=False, *, attention_mode=AttentionMode.SORT_BASED_LINEAR):
+        assert codebook.shape[1] % 128 == 0
+        self.window_length = window_length
+        self.codebook = codebook
+        self.sphere = sphere
+        self.attention_mode = attention_mode
+        self.key_codes = []    # per layer: [B,H,N,1] uint8 (only when the codebook has <= 256 entries)
+        self.value_cache = []  # per layer: [B,H,N,D]
+        self.seen_tokens = 0
+
+    def get_seq_length(self, layer_idx=0):
+        return 0 if len(self.value_cache) <= layer_idx else self.value_cache[layer_idx].shape[-2]
+
+
+def rotate_half(x):
+    half = x.shape[-1] // 2
+    return torch.cat((-x[..., half:], x[..., :half]), dim=-1)
+
+
+def rope_tables(head_dim, n_pos, base=10000.0, dtype=torch.float32, device=None):
+    """cos / sin [n_pos, D] of the transformers ~4.37 rotary embedding the reference's modules call
+    (inv_freq = base^(-2r/D), emb = cat(freqs, freqs)), cast to the model dtype."""
+    inv_freq = 1.0 / (base ** (torch.arange(0, head_dim, 2, dtype=torch.float32, device=device) / head_dim))
+    freqs = torch.outer(torch.arange(n_pos, dtype=torch.float32, device=device), inv_freq)
+    emb = torch.cat((freqs, freqs), dim=-1)
+    return emb.cos().to(dtype), emb.sin().to(dtype)
+
+
+def rerope_operands(query_states, key_states, position_ids, window_length, rope_base=10000.0):
+    """(q1, k1, q2) of ops/attn_vq.py:402-407: rotary at the true positions, and the query at the clamped position
+    window_length + 1.  position_ids [B,N]; states [B,H,N,D]."""
+    B, H, N, D = query_states.shape
+    n_pos = max(int(position_ids.max()) + 1, window_length + 2)
+    cos, sin = rope_tables(D, n_pos, rope_base, query_states.dtype, query_states.device)
+    c, s = cos[position_ids].unsqueeze(1), sin[position_ids].unsqueeze(1)  # [B,1,N,D]
+    q1 = query_states * c + rotate_half(query_states) * s
+    k1 = key_states * c + rotate_half(key_states) * s
+    cw, sw = cos[window_length + 1], sin[window_length + 1]
+    q2 = query_states * cw + rotate_half(query_states) * sw
+    return q1, k1, q2
+
+
+def sort_based_preprocess(vq_key_ids, vq_key_onehot, value_states, block=BLOCK_SIZE):
+    """Inputs of the count kernel from the key codes, following ops/attn_vq.py:352-384, 410-413: running per-code key
+    counts, V sorted by (code, position) with per-code prefix sums (fp32 cumsum, cast to the model dtype), and the
+    prefix-sum row index per (block, code).  Returns (k_vq_cnt [B,H,N//block,C] int64, v_vq [B,H,N+1,D],
+    vi [B,H,N//block,C] int64)."""
+    B, H, N = vq_key_ids.shape
+    D = value_states.shape[-1]
+    dtype, device = value_states.dtype, value_states.device
+    assert vq_key_onehot.shape[-1] < (1 << 13) and N < (1 << 18)
+    cum = torch.cumsum(vq_key_onehot, dim=2)
+    order = ((vq_key_ids.to(torch.int32) << 18) + torch.arange(N, dtype=torch.int32, device=device)).argsort()
+    v_vq = torch.zeros((B, H, N + 1, D), device=device, dtype=torch.float32)
+    v_vq[:, :, 1:] = torch.gather(value_states, 2, order[..., None].expand(-1, -1, -1, D)).float()
+    v_vq = torch.cumsum(v_vq, 2)
+    total = cum[:, :, -1]
+    start = torch.cumsum(total, dim=-1) - total
+    seg_base = v_vq.gather(2, start[..., None].expand(-1, -1, -1, D))
+    code_sorted = torch.gather(vq_key_ids, 2, order)
+    v_vq[:, :, 1:] -= seg_base.gather(2, code_sorted[..., None].expand(-1, -1, -1, D))
+    vi = cum + start[:, :, None, :]
+    return cum[:, :, block - 1::block].contiguous(), v_vq.to(dtype), vi[:, :, block - 1::block].contiguous()
+
+
+def long_prefilling_sort_based_linear(query_states, key_states, value_states, position_ids, cache, layer_idx=0,
+                                      rope_base=10000.0):
+    """Linear-time prefill with VQ memory (ops/attn_vq.py:336-443): encode keys with the head's codebook, build the
+    count-kernel inputs, run `vq_attn_forward`.  States [B,H,N,D]; returns [B, N, H*D] like the reference (no o_proj)."""
+    from .triton_fused_vq_attn import vq_attn_forward
+
+    B, H, N, D = query_states.shape
+    dtype = query_states.dtype
+    _, ids, onehot = multi_head_single_quantize(key_states, cache.codebook)
+    cnt, v_vq, vi = sort_based_preprocess(ids, onehot, value_states)
+    q1, k1, q2 = rerope_operands(query_states, key_states, position_ids, cache.window_length, rope_base)
+    out = vq_attn_forward(q1, q2, k1, cache.codebook, cnt.to(dtype), key_states, value_states, v_vq, vi,
+                          cache.window_length, softmax_scale=1 / math.sqrt(D))
+    _remember(cache, layer_idx, ids, value_states, N)
+    return out.transpose(1, 2).contiguous().flatten(2)
+
+
+def long_prefilling_per_key(query_states, key_states, value_states, position_ids, cache, layer_idx=0,
+                            rope_base=10000.0):
+    """Same result through the fused per-key kernel (`attn_vq_prefill` with M = 1): no one-hot cumsum, no sort, no
+    merge pass.  Needs a codebook of at most 256 entries (uint8 codes)."""
+    B, H, N, D = query_states.shape
+    assert cache.codebook.shape[1] <= 256
+    _, ids, _ = multi_head_single_quantize(key_states, cache.codebook)
+    q1, k1, q2 = rerope_operands(query_states, key_states, position_ids, cache.window_length, rope_base)
+    out = attn_vq_prefill(q1, ids.to(torch.uint8).unsqueeze(-1), cache.codebook.unsqueeze(1), value_states,
+                          k_exact=k1, window_size=cache.window_length, q2=q2, k2=key_states,
+                          softmax_scale=1 / math.sqrt(D))
+    _remember(cache, layer_idx, ids, value_states, N)
+    return out.transpose(1, 2).contiguous().flatten(2)
+
+
+def _remember(cache, layer_idx, ids, value_states, n_tokens):
+    if layer_idx == 0:
+        cache.seen_tokens += n_tokens
+    if len(cache.value_cache) <= layer_idx and cache.codebook.shape[1] <= 256:
+        cache.key_codes.append(ids.to(torch.uint8).unsqueeze(-1).contiguous())
+        cache.value_cache.append(value_states)
+
+
+def long_prefilling_slow_reference_impl(query_states, key_states, value_states, position_ids, cache, rope_base=10000.0):
+    """Per-query loops of ops/attn_vq.py:278-334, kept for checking the linear-time path (torch ops, any device)."""
+    B, H, N, D = query_states.shape
+    W = cache.window_length
+    q1, k1, q2 = rerope_operands(query_states, key_states, position_ids, W, rope_base)
+    k_hat, _, _ = multi_head_single_quantize(key_states, cache.codebook)
+    scale = 1.0 / math.sqrt(D)
+    output = torch.zeros_like(query_states, memory_format=torch.contiguous_format)
+    for b in range(B):
+        for h in range(H):
+            for qi in range(N):
+                boundary = max(0, (qi - W) // BLOCK_SIZE * BLOCK_SIZE)
+                local_boundary = max(0, qi - W)
+                attn = [q1[b, h, qi] @ k1[b, h, local_boundary:qi + 1].T]
+                v = [value_states[b, h, local_boundary:qi + 1]]
+                if local_boundary > 0:
+                    attn.append(q2[b, h, qi] @ key_states[b, h, boundary:local_boundary].T)
+                    v.append(value_states[b, h, boundary:local_boundary])
+                if boundary > 0:
+                    attn.append(q2[b, h, qi] @ k_hat[b, h, :boundary].T)
+                    v.append(value_states[b, h, :boundary])
+                w = torch.softmax(torch.cat(attn).float() * scale, dim=0).to(value_states.dtype)
+                output[b, h, qi] = w @ torch.cat(v)
+    return output.transpose(1, 2).contiguous().flatten(2)
+
+
+def dispatch_attn(query_states, key_states, value_states, position_ids, cache, layer_idx=0, rope_base=10000.0):
+    """Routing of `_dispatch_attn_impl` (ops/attn_vq.py:225-248): a prefill longer than window + 128 goes to the
+    VQ-memory path chosen by `cache.attention_mode`; a shorter prefill is plain causal attention on the rotated
+    operands; a seqlen_q == 1 step attends over the cached codes (the route the reference leaves unimplemented)."""
+    from .triton_fused_local_attn import flash_attn_func as causal_window_attention
+
+    B, H, q_len, D = query_states.shape
+    is_prefilling = cache.get_seq_length(layer_idx) == 0
+    if is_prefilling and q_len > cache.window_length + BLOCK_SIZE:
+        if cache.attention_mode == AttentionMode.SORT_BASED_LINEAR:
+            return long_prefilling_sort_based_linear(query_states, key_states, value_states, position_ids, cache,
+                                                     layer_idx, rope_base)
+        if cache.attention_mode == AttentionMode.SLOW_REFERNECE:
+            return long_prefilling_slow_reference_impl(query_states, key_states, value_states, position_ids, cache,
+                                                       rope_base)
+        raise KeyError(f"Bad attention mode: {cache.attention_mode}")
+    if is_prefilling:
+        q1, k1, _ = rerope_operands(query_states, key_states, position_ids, cache.window_length, rope_base)
+        out = causal_window_attention(q1.transpose(1, 2), k1.transpose(1, 2), value_states.transpose(1, 2), q_len,
+                                      softmax_scale=1 / math.sqrt(D))
+        _, ids, _ = multi_head_single_quantize(key_states, cache.codebook)
+        _remember(cache, layer_idx, ids, value_states, q_len)
+        return out.contiguous().flatten(2)
+    assert q_len == 1, "Only support prefilling or generation"
+    assert len(cache.key_codes) > layer_idx, "decode needs a codebook of at most 256 entries"
+    # generation step: append the new key's code and value, then attend over all codes with the clamped query
+    _, ids, _ = multi_head_single_quantize(key_states, cache.codebook)
+    cache.key_codes[layer_idx] = torch.cat([cache.key_codes[layer_idx], ids.to(torch.uint8).unsqueeze(-1)], dim=2)
+    cache.value_cache[layer_idx] = torch.cat([cache.value_cache[layer_idx], value_states], dim=2)
+    if layer_idx == 0:
+        cache.seen_tokens += 1
+    cos, sin = rope_tables(D, cache.window_length + 2, rope_base, query_states.dtype, query_states.device)
+    q2 = query_states * cos[cache.window_length + 1] + rotate_half(query_states) * sin[cache.window_length + 1]
+    out = attn_vq_decode(q2, cache.key_codes[layer_idx], cache.codebook.unsqueeze(1), cache.value_cache[layer_idx],
+                         softmax_scale=1 / math.sqrt(D))
+    return out.transpose(1, 2).contiguous().flatten(2)
