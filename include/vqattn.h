@@ -149,6 +149,17 @@ int vqa_prefill_f16(const void* q, const uint8_t* codes, const void* codebooks, 
                     int B, int H, int N, int D, int M, int K, const int64_t* strides, int window, int boundary_mode,
                     int causal, float sm_scale, vqa_stream_t stream);
 
+/* fp32 validation instantiation of the prefill: every visible key quantised (no exact window), plain fp32 FMA
+ * arithmetic with the lookup-table formulation (LUT[i,m,c] = <q_i, codebooks[h,m,c]>, score = sum_m LUT[i,m,code_jm]);
+ * checks the additive-code attention against a dense fp32 softmax to 1e-4.  q, v, out float [B,H,N,D]-addressable,
+ * codebooks float [H,M,K,D]; strides[0..13]: q(b,h,n) codes(b,h) codebooks(h,m,k) v(b,h,n) out(b,h,n).  M <= 8.
+ * Counterpart of the fp32 branch of the naive reference (softmax in fp32, ops/attn_vq.py:331). */
+#define VQA_PREFILL_F32_NUM_STRIDES 14
+
+int vqa_prefill_f32(const float* q, const uint8_t* codes, const float* codebooks, const float* v, float* out,
+                    float* lse, int B, int H, int N, int D, int M, int K, const int64_t* strides, int causal,
+                    float sm_scale, vqa_stream_t stream);
+
 /* ------------------------------------------------------------------------------------------------------------------
  * Count-weighted far-context kernel of the single-codebook formulation.  Replaces _vq_fwd_kernel
  * (ops/triton_fused_vq_attn.py:88-187) including the host-side zero / -inf initialisation (:214-215):

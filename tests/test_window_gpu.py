@@ -235,3 +235,22 @@ def test_count_kernel_and_merge_separately():
     torch.cuda.synchronize()
     assert_close_16(a, want_m, "merge")
     assert_close_lse(sa, want_s)
+
+
+# ------------------------------------------------------------------ fp32 validation instantiation
+@pytest.mark.parametrize("B,H,N,D,M,K,causal", [(1, 8, 1024, 64, 2, 256, True), (2, 2, 333, 128, 4, 256, True),
+                                                 (1, 2, 1500, 64, 1, 100, False), (1, 1, 70, 128, 8, 256, True)])
+def test_vq_prefill_fp32_config1(B, H, N, D, M, K, causal):
+    """BASELINE configuration 1 (batch 1, 8 heads, 1024 tokens, head_dim 64, fp32, 2 x 256 codebooks ~N(0, 0.5)) and
+    variations, against the naive softmax(Q K_hat^T / sqrt(d)) V to 1e-4."""
+    _say(f"vq prefill fp32 B{B} H{H} N{N} D{D} M{M} K{K} causal={causal}")
+    g = torch.Generator("cpu").manual_seed(1)
+    q, v = torch.randn(B, H, N, D, generator=g), torch.randn(B, H, N, D, generator=g)
+    cb = torch.randn(H, M, K, D, generator=g) * 0.5
+    codes = torch.randint(0, K, (B, H, N, M), generator=g, dtype=torch.int32).to(torch.uint8)
+    want, want_lse = oracle.attn_vq_prefill(q, codes, cb, v, causal=causal)
+    out, lse = attn_vq_prefill(q.cuda(), codes.cuda(), cb.cuda(), v.cuda(), causal=causal, return_lse=True)
+    torch.cuda.synchronize()
+    assert out.dtype == torch.float32
+    assert (out.cpu() - want).abs().max() <= 1e-4
+    assert (lse.cpu() - want_lse).abs().max() <= 1e-4

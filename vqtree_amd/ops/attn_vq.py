@@ -89,6 +89,8 @@ def attn_vq_prefill(q, k_codes, codebooks, v, *, k_exact=None, window_size=0, ca
     assert codebooks.shape == (H, M, K, D), "codebooks must be [H,M,K,D]"
     assert v.shape == (B, H, N, D), "seqlen_q == seqlen_k prefill only"
     assert causal or k_exact is None, "non-causal attention takes quantised keys only"
+    if q.dtype == torch.float32:
+        return _attn_vq_prefill_f32(q, k_codes, codebooks, v, k_exact, q2, k2, causal, softmax_scale, return_lse)
     sfx = check_same_16bit(q, codebooks, v, k_exact, q2, k2)
     q, codebooks, v, k_exact, q2, k2 = last_dim_contiguous(q, codebooks, v, k_exact, q2, k2)
     if k_codes.stride(3) != 1 or k_codes.stride(2) != M:
@@ -112,6 +114,30 @@ def attn_vq_prefill(q, k_codes, codebooks, v, *, k_exact=None, window_size=0, ca
             ptr(q), ptr(k_codes), ptr(codebooks), ptr(v), ptr(k_exact), ptr(q2), ptr(k2), ptr(out), ptr(lse),
             ptr(workspace), ws_bytes, B, H, N, D, M, K, strides, int(window_size), BOUNDARY[boundary_mode],
             1 if causal else 0, softmax_scale, _lib.current_stream(q.device))
+    _lib.check(rc)
+    return (out, lse) if return_lse else out
+
+
+def _attn_vq_prefill_f32(q, k_codes, codebooks, v, k_exact, q2, k2, causal, softmax_scale, return_lse):
+    """fp32 validation path: every visible key quantised (no exact window), plain fp32 arithmetic."""
+    from ._common import bhn_strides, last_dim_contiguous, ptr
+
+    assert k_exact is None and q2 is None and k2 is None, "the fp32 path takes quantised keys only"
+    assert q.dtype == codebooks.dtype == v.dtype == torch.float32, "All tensors must have the same type"
+    lib = _lib.load()
+    B, H, N, D = q.shape
+    M, K = k_codes.shape[3], codebooks.shape[2]
+    q, codebooks, v = last_dim_contiguous(q, codebooks, v)
+    if k_codes.stride(3) != 1 or k_codes.stride(2) != M:
+        k_codes = k_codes.contiguous()
+    out = torch.empty((B, H, N, D), dtype=torch.float32, device=q.device)
+    lse = torch.empty((B, H, N), dtype=torch.float32, device=q.device) if return_lse else None
+    strides = _lib.strides_array(*bhn_strides(q), k_codes.stride(0), k_codes.stride(1), codebooks.stride(0),
+                                 codebooks.stride(1), codebooks.stride(2), *bhn_strides(v), *bhn_strides(out))
+    with torch.cuda.device(q.device):
+        rc = lib.vqa_prefill_f32(ptr(q), ptr(k_codes), ptr(codebooks), ptr(v), ptr(out), ptr(lse), B, H, N, D, M, K,
+                                 strides, 1 if causal else 0, softmax_scale or 1.0 / math.sqrt(D),
+                                 _lib.current_stream(q.device))
     _lib.check(rc)
     return (out, lse) if return_lse else out
 
