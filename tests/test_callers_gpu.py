@@ -88,3 +88,35 @@ def test_short_prefill_then_generation_steps():
         q2 = qs * cos[W + 1] + A.rotate_half(qs) * sin[W + 1]
         want, _ = oracle.attn_vq_decode(q2, cache.key_codes[0], cb.unsqueeze(1), cache.value_cache[0], 1 / math.sqrt(D))
         assert_close_16(o.view(B, 1, H, D).transpose(1, 2), want, f"generation step {step}")
+
+
+def test_decode_harness_matches_dense_reference():
+    """Small Llama-shaped decode loop over a VQ key cache: the HIP decode kernel inside the loop against dense fp32
+    attention over the reconstructed keys, step by step on identical state."""
+    from vqtree_amd.decode_harness import VQDecodeModel, encode_residual
+
+    def dense_attention(q2, codes, codebooks, v, softmax_scale):
+        out, _ = oracle.attn_vq_decode(q2, codes, codebooks, v, softmax_scale)
+        return out.to(q2.dtype).cuda()
+
+    kw = dict(layers=2, hidden=256, heads=2, head_dim=128, ffn=512, vocab=1000, n_codebooks=4, window=128,
+              capacity=400, batch=2)
+    a, b = VQDecodeModel(**kw), VQDecodeModel(**kw)
+    a.fill_random_context(300), b.fill_random_context(300)
+    tok = torch.tensor([3, 777], device="cuda")
+    for step in range(3):
+        ta, la = a.step(tok, return_logits=True)
+        tb, lb = b.step(tok, attention=dense_attention, return_logits=True)
+        assert (la.float() - lb.float()).abs().max() <= 2e-2 * max(1.0, float(lb.float().abs().max()))
+        assert torch.equal(a.layers[0]["codes"][:, :, 300 + step], b.layers[0]["codes"][:, :, 300 + step])
+        tok = tb
+    assert a.length == 303
+    # the greedy residual encoder picks, stage by stage, the nearest codeword of the running residual
+    x = torch.randn(1, 2, 5, 128, device="cuda")
+    cb = a.layers[0]["codebooks"]
+    codes = encode_residual(x, cb)
+    r = x[0, 1, 2].float()
+    for m in range(4):
+        d = ((r[None] - cb[1, m].float()) ** 2).sum(-1)
+        assert int(codes[0, 1, 2, m]) == int(d.argmin())
+        r = r - cb[1, m, int(codes[0, 1, 2, m])].float()

@@ -1,0 +1,159 @@
+"""Llama-shaped greedy decode loop over a VQ-coded key cache (counterpart of the reference's generation demo `gen.py`
+and of the seqlen_q == 1 branch of its attention module, ops/attn_vq.py:176-223, which the reference leaves
+unimplemented).
+
+Every layer keeps, per (batch, head): the additive-quantiser codes of its keys `[B,H,cap,M] uint8` and the values
+`[B,H,cap,D]`.  A step projects the new token, rotates q to the clamped ReRoPE position, encodes the new key greedily
+against the layer's codebooks (residual, nearest codeword), appends code and value, and attends over the whole cache
+with the HIP decode kernel.  The linear layers are plain torch matmuls (weights ~ N(0, 0.02)): they are plumbing around
+the attention path, which is what this harness measures.
+
+    python -m vqtree_amd.decode_harness --layers 32 --context 65536 --batch 4 --steps 128
+"""
+import argparse
+import json
+import math
+import time
+
+import torch
+
+from .ops.attn_vq import attn_vq_decode, rope_tables, rotate_half
+
+
+def encode_residual(x, codebooks):
+    """Greedy additive (residual) encoding: code_m = argmin_c |r - cb[h,m,c]|^2, r -= cb[h,m,code_m].
+
+    x [B,H,T,D], codebooks [H,M,K,D] -> codes [B,H,T,M] uint8.  fp32 arithmetic."""
+    r = x.float()
+    cb = codebooks.float()
+    half_norm = 0.5 * (cb * cb).sum(-1)  # [H,M,K]
+    codes = []
+    for m in range(cb.shape[1]):
+        score = torch.einsum("bhtd,hkd->bhtk", r, cb[:, m]) - half_norm[:, m][None, :, None, :]
+        idx = score.argmax(-1)  # nearest codeword in L2
+        codes.append(idx)
+        picked = cb[:, m].unsqueeze(0).expand(r.shape[0], -1, -1, -1).gather(
+            2, idx.unsqueeze(-1).expand(-1, -1, -1, r.shape[-1]))
+        r = r - picked
+    return torch.stack(codes, dim=-1).to(torch.uint8)
+
+
+class VQDecodeModel:
+    """Random-init Llama-2-shaped decoder (RMSNorm, rotary attention over a VQ key cache, SwiGLU MLP)."""
+
+    def __init__(self, layers, hidden, heads, head_dim, ffn, vocab, n_codebooks, window, capacity, batch,
+                 dtype=torch.bfloat16, device="cuda", seed=5, cb_std=0.35):
+        g = torch.Generator(device=device).manual_seed(seed)
+        w = lambda *s: (torch.randn(*s, generator=g, device=device, dtype=torch.float32) * 0.02).to(dtype)
+        self.L, self.hidden, self.H, self.D, self.M = layers, hidden, heads, head_dim, n_codebooks
+        self.window, self.capacity, self.B = window, capacity, batch
+        self.dtype, self.device = dtype, device
+        self.embed = w(vocab, hidden)
+        self.lm_head = w(hidden, vocab)
+        self.layers = []
+        for _ in range(layers):
+            self.layers.append(dict(
+                wqkv=w(hidden, 3 * heads * head_dim), wo=w(heads * head_dim, hidden),
+                w_gate_up=w(hidden, 2 * ffn), w_down=w(ffn, hidden),
+                codebooks=(torch.randn(heads, n_codebooks, 256, head_dim, generator=g, device=device) * cb_std).to(dtype),
+                codes=torch.empty(batch, heads, capacity, n_codebooks, dtype=torch.uint8, device=device),
+                values=torch.empty(batch, heads, capacity, head_dim, dtype=dtype, device=device),
+            ))
+        self.length = 0
+        cos, sin = rope_tables(head_dim, window + 2, dtype=dtype, device=device)
+        self.cos_w, self.sin_w = cos[window + 1], sin[window + 1]  # every far key is seen at the clamped position
+
+    def fill_random_context(self, n_tokens, seed=6):
+        """Synthetic cache contents standing in for a prefill of n_tokens (random codes, V ~ N(0,1))."""
+        g = torch.Generator(device=self.device).manual_seed(seed)
+        for layer in self.layers:
+            layer["codes"][:, :, :n_tokens] = torch.randint(0, 256, (self.B, self.H, n_tokens, self.M), generator=g,
+                                                            device=self.device, dtype=torch.uint8)
+            for b in range(self.B):
+                layer["values"][b, :, :n_tokens] = torch.randn(self.H, n_tokens, self.D, generator=g,
+                                                               device=self.device).to(self.dtype)
+        self.length = n_tokens
+
+    @staticmethod
+    def _rms(x):
+        return (x.float() * torch.rsqrt(x.float().pow(2).mean(-1, keepdim=True) + 1e-5)).to(x.dtype)
+
+    def step(self, tokens, attention=None, return_logits=False, events=None):
+        """One greedy decode step for token ids [B]; returns next token ids [B] (and the logits).  `attention`
+        overrides the attention operator (tests pass a dense reference)."""
+        attention = attention or attn_vq_decode
+        B, H, D = self.B, self.H, self.D
+        n = self.length
+        x = self.embed[tokens]  # [B, hidden]
+        for layer in self.layers:
+            h = self._rms(x)
+            qkv = (h @ layer["wqkv"]).view(B, 3, H, D)
+            q, k, v = qkv[:, 0], qkv[:, 1], qkv[:, 2]  # [B,H,D]
+            q2 = (q * self.cos_w + rotate_half(q) * self.sin_w).unsqueeze(2)  # [B,H,1,D]
+            layer["codes"][:, :, n] = encode_residual(k.unsqueeze(2), layer["codebooks"])[:, :, 0]
+            layer["values"][:, :, n] = v
+            if events is not None:
+                events.append(torch.cuda.Event(enable_timing=True))
+                events[-1].record()
+            o = attention(q2, layer["codes"][:, :, : n + 1], layer["codebooks"], layer["values"][:, :, : n + 1],
+                          softmax_scale=1.0 / math.sqrt(D))
+            if events is not None:
+                events.append(torch.cuda.Event(enable_timing=True))
+                events[-1].record()
+            x = x + o.reshape(B, H * D) @ layer["wo"]
+            h = self._rms(x)
+            gate, up = (h @ layer["w_gate_up"]).chunk(2, dim=-1)
+            x = x + (torch.nn.functional.silu(gate) * up) @ layer["w_down"]
+        self.length = n + 1
+        logits = self._rms(x) @ self.lm_head
+        return (logits.argmax(-1), logits) if return_logits else logits.argmax(-1)
+
+    def attention_bytes_per_step(self):
+        """Algorithmic bytes of the attention path per token step: per layer codes + V + codebooks + q/out."""
+        e = 2
+        n = self.length
+        per_layer = self.B * self.H * n * self.M + e * self.B * self.H * n * self.D + e * self.H * self.M * 256 * self.D \
+            + 2 * e * self.B * self.H * self.D
+        return self.L * per_layer
+
+
+def run(layers=32, hidden=4096, heads=32, head_dim=128, ffn=11008, vocab=32000, n_codebooks=4, context=65536, batch=4,
+        steps=128, warmup=4, window=1024, device="cuda"):
+    model = VQDecodeModel(layers, hidden, heads, head_dim, ffn, vocab, n_codebooks, window, context + steps + warmup,
+                          batch, device=device)
+    model.fill_random_context(context)
+    g = torch.Generator(device=device).manual_seed(7)
+    tokens = torch.randint(0, vocab, (batch,), generator=g, device=device)
+    with torch.no_grad():
+        for _ in range(warmup):
+            tokens = model.step(tokens)
+        torch.cuda.synchronize()
+        bytes_mid = None
+        events = []
+        t0 = time.perf_counter()
+        for s in range(steps):
+            if s == steps // 2:
+                bytes_mid = model.attention_bytes_per_step()
+            tokens = model.step(tokens, events=events)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+    us = dt / steps * 1e6
+    attn_us = sum(events[i].elapsed_time(events[i + 1]) for i in range(0, len(events), 2)) / steps * 1e3
+    return {
+        "workload": f"{layers}-layer Llama-2-7B-shaped greedy decode, batch {batch}, context {context}, VQ key cache "
+                    f"{n_codebooks}x256 per layer, {steps} steps",
+        "us_per_step": round(us, 1),
+        "attention_us_per_step": round(attn_us, 1),
+        "attention_bytes_per_step": bytes_mid,
+        "attention_GBps": round(bytes_mid / (attn_us * 1e-6) / 1e9, 1),
+        "attention_hbm_frac": round(bytes_mid / (attn_us * 1e-6) / 8e12, 4),
+        "note": "us_per_step is whole-step wall time (projections, MLP, key encoder, attention); attention_us_per_step "
+                "sums HIP-event intervals around the attention calls of all layers (3 kernels each)",
+    }
+
+
+if __name__ == "__main__":
+    ap = argparse.ArgumentParser()
+    for name, default in (("layers", 32), ("context", 65536), ("batch", 4), ("steps", 128), ("warmup", 4)):
+        ap.add_argument("--" + name, type=int, default=default)
+    print(json.dumps(run(**vars(ap.parse_args()))))
