@@ -195,6 +195,52 @@ int vqa_merge_state_inplace_bf16(void* o, float* s, const void* o_other, const f
 int vqa_merge_state_inplace_f16(void* o, float* s, const void* o_other, const float* s_other, int B, int H, int N,
                                 int D, const int64_t* strides, vqa_stream_t stream);
 
+/* ------------------------------------------------------------------------------------------------------------------
+ * Key encoder: nearest-codeword search of every key against its head's codebooks.
+ *   mode 0: id_m = argmax_c <x, codebooks[h,m,c]> for every codebook m independently (inner product, first maximum
+ *           on ties) -- replaces multi_head_single_quantize, ops/mini_vq.py:4-18 (M = 1); with round_scores != 0 the
+ *           scores are rounded to the element type before the comparison, like the reference's einsum in the model
+ *           dtype (ops/mini_vq.py:10-11).
+ *   mode 1: greedy residual (additive) encoding in the L2 sense: r = x; id_m = argmax_c (<r, cb[h,m,c]> - |cb|^2/2);
+ *           r -= cb[h,m,id_m].  Produces the [B,H,N,M] codes of vqa_decode / vqa_prefill; the reference trains such
+ *           codebooks offline (build_quantizer/120_build_additive_quantizer.py:23-32) and has no runtime encoder.
+ *
+ *   x [B,H,N,D]; codebooks [H,M,K,D], K % 32 == 0; codes [B,H,N,M] uint8 (nullable, needs K <= 256);
+ *   ids [B,H,N,M] int64 (nullable); at least one output.  D in {16,32,64,128}.
+ *   strides[0..11] = x(b,h,n) codebooks(h,m,k) codes(b,h,n) ids(b,h,n); m is innermost in codes and ids.
+ * ------------------------------------------------------------------------------------------------------------------ */
+#define VQA_ENCODE_NUM_STRIDES 12
+
+int vqa_encode_keys_bf16(const void* x, const void* codebooks, uint8_t* codes, int64_t* ids, int B, int H, int N, int D,
+                         int M, int K, const int64_t* strides, int mode, int round_scores, vqa_stream_t stream);
+
+int vqa_encode_keys_f16(const void* x, const void* codebooks, uint8_t* codes, int64_t* ids, int B, int H, int N, int D,
+                        int M, int K, const int64_t* strides, int mode, int round_scores, vqa_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------------------------------
+ * Inputs of vqa_vqcount_fwd from per-key code ids -- replaces the one-hot cumulative sum, argsort and global prefix
+ * sum of ops/attn_vq.py:352-384 and the block sampling at :410-413:
+ *   cnt[t,c] = #{j < (t+1)*128 : id_j == c}, t < N/128;   vi[t,c] = cnt[t,c] + #{j < N : id_j < c};
+ *   v_vq[0] = 0, v_vq[1+r] = running sum of V over the keys of r's code in (code, position) order up to row r
+ *   (fp32 running sum per code, rounded to the element type).
+ *
+ *   ids [B,H,N] int64 (values outside [0, C) are clamped); v [B,H,N,D]; cnt [B,H,N/128,C] int64 (nullable);
+ *   cnt_elem: the same counts in the element type, as vqa_vqcount_fwd reads them (nullable); v_vq [B,H,N+1,D];
+ *   vi [B,H,N/128,C] int64 (may be null when N < 128).  C <= 8192, D even and <= 128.
+ *   strides[0..17] = ids(b,h,n) v(b,h,n) cnt(b,h,t) cnt_elem(b,h,t) v_vq(b,h,n) vi(b,h,t).
+ * ------------------------------------------------------------------------------------------------------------------ */
+#define VQA_PREPROCESS_NUM_STRIDES 18
+
+size_t vqa_preprocess_workspace_bytes(int B, int H, int N, int C);
+
+int vqa_preprocess_bf16(const int64_t* ids, const void* v, int64_t* cnt, void* cnt_elem, void* v_vq, int64_t* vi,
+                        void* workspace, size_t workspace_bytes, int B, int H, int N, int D, int C,
+                        const int64_t* strides, vqa_stream_t stream);
+
+int vqa_preprocess_f16(const int64_t* ids, const void* v, int64_t* cnt, void* cnt_elem, void* v_vq, int64_t* vi,
+                       void* workspace, size_t workspace_bytes, int B, int H, int N, int D, int C,
+                       const int64_t* strides, vqa_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -16,6 +16,8 @@ Pinning status (see tests/test_oracle_pins.py):
   * count-based far kernel + sort preprocessing  : pinned (brute-force segment sums, M=1 identity with the
                                                    per-key formulation)
   * multi_head_single_quantize                   : pinned (brute-force argmax, first-max tie rule)
+  * encode_residual (greedy additive encoder)    : pinned (brute-force nearest neighbour per stage; no reference
+                                                   counterpart exists at run time)
 """
 from .attention import (  # noqa: F401
     LOG2E,
@@ -34,6 +36,7 @@ from .attention import (  # noqa: F401
 )
 from .rope import apply_rope, rope_tables, rotate_half  # noqa: F401
 from .vq import (  # noqa: F401
+    encode_residual,
     multi_head_single_quantize,
     reconstruct_keys,
     sort_based_preprocess,

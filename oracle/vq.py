@@ -40,6 +40,28 @@ def multi_head_single_quantize(inp, codebook):
     return quant, ids, onehot
 
 
+def encode_residual(x, codebooks):
+    """Greedy additive (residual) encoder: r = x; for every codebook m: id_m = argmin_c |r - cb[h,m,c]|^2 (first
+    minimum on ties), evaluated as argmax_c (<r, c> - |c|^2 / 2) in fp32; r -= cb[h,m,id_m].
+
+    The reference has no runtime encoder for additive codes (its codebooks come from the offline faiss trainer,
+    build_quantizer/120_build_additive_quantizer.py:23-32); this is the textbook greedy residual search, pinned by
+    brute-force nearest-neighbour search in tests/test_oracle_pins.py.
+    x [B,H,N,D], codebooks [H,M,K,D] -> codes [B,H,N,M] int64.
+    """
+    r = _f32(x).clone()
+    cb = _f32(codebooks)
+    B, H, N, D = r.shape
+    out = torch.zeros(B, H, N, cb.shape[1], dtype=torch.int64)
+    for m in range(cb.shape[1]):
+        for h in range(H):
+            score = r[:, h] @ cb[h, m].T - 0.5 * (cb[h, m] * cb[h, m]).sum(-1)
+            idx = score.argmax(-1)
+            out[:, h, :, m] = idx
+            r[:, h] -= cb[h, m][idx]
+    return out
+
+
 def sort_based_preprocess(ids, v, n_codes, dtype=None, block=T_BLOCK):
     """Inputs of the count kernel, following ops/attn_vq.py:352-384 and the block sampling at :410-413.
 

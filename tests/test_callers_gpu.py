@@ -112,7 +112,7 @@ def test_decode_harness_matches_dense_reference():
         tok = tb
     assert a.length == 303
     # the greedy residual encoder picks, stage by stage, the nearest codeword of the running residual
-    x = torch.randn(1, 2, 5, 128, device="cuda")
+    x = torch.randn(1, 2, 5, 128, device="cuda").bfloat16()
     cb = a.layers[0]["codebooks"]
     codes = encode_residual(x, cb)
     r = x[0, 1, 2].float()
@@ -120,3 +120,46 @@ def test_decode_harness_matches_dense_reference():
         d = ((r[None] - cb[1, m].float()) ** 2).sum(-1)
         assert int(codes[0, 1, 2, m]) == int(d.argmin())
         r = r - cb[1, m, int(codes[0, 1, 2, m])].float()
+
+
+def test_rerope_caller_routes():
+    """Attention core of the ReRoPE module: long prefill through the full ReRoPE kernel against the dense oracle,
+    cache contents after it, a short prefill (plain causal) and a generation step against dense softmax over the
+    cached keys."""
+    from vqtree_amd.ops.attn_rerope import ReRoPECache, rerope_attn_forward
+    from vqtree_amd.ops.attn_vq import rope_tables, rotate_half
+
+    print("callers: rerope module core, N=300 W=128", flush=True)
+    B, H, N, D, W = 1, 4, 300, 64, 128
+    q, k, v = _states(B, H, N, D, torch.bfloat16, 11)
+    pos = torch.arange(N, device="cuda").unsqueeze(0)
+    cache = ReRoPECache(W)
+    out = rerope_attn_forward(q, k, v, pos, cache)
+    torch.cuda.synchronize()
+    assert out.shape == (B, N, H * D)
+    cos, sin = rope_tables(D, N + 1, dtype=torch.bfloat16, device="cuda")
+    rope = lambda x, p: x * cos[p] + rotate_half(x) * sin[p]
+    q1, k1, q2 = rope(q, pos[0]), rope(k, pos[0]), rope(q, W)
+    ref, _ = oracle.rerope_full(q1.cpu(), q2.cpu(), k1.cpu(), k.cpu(), v.cpu(), True, 1 / math.sqrt(D), W)
+    assert_close_16(out.view(B, N, H, D).transpose(1, 2).cpu(), ref)
+    assert cache.get_seq_length() == N
+    assert torch.equal(cache.key_cache[0][:, :, -W:], k1[:, :, -W:])
+    assert torch.equal(cache.key_cache[0][:, :, :-W], rope(k, N - W)[:, :, :-W])
+
+    # generation step: dense softmax over the keys the cache returns after the append
+    g = torch.Generator("cpu").manual_seed(12)
+    qn, kn, vn = (torch.randn(B, H, 1, D, generator=g).bfloat16().cuda() for _ in range(3))
+    step = rerope_attn_forward(qn, kn, vn, torch.tensor([[N]], device="cuda"), cache)
+    keys, vals = cache.key_cache[0].float().cpu(), cache.value_cache[0].float().cpu()
+    cos2, sin2 = rope_tables(D, N + 1, dtype=torch.bfloat16, device="cuda")
+    qr = (qn * cos2[N] + rotate_half(qn) * sin2[N]).float().cpu()
+    want = torch.softmax(qr @ keys.transpose(-1, -2) / math.sqrt(D), -1) @ vals
+    assert cache.get_seq_length() == N + 1
+    assert_close_16(step.view(B, 1, H, D).transpose(1, 2).cpu(), want)
+
+    # short prefill: window covers everything -> causal attention on the rotated operands
+    Ns = 100
+    short = rerope_attn_forward(q[:, :, :Ns], k[:, :, :Ns], v[:, :, :Ns], pos[:, :Ns], ReRoPECache(W))
+    scores = q1[:, :, :Ns].float().cpu() @ k1[:, :, :Ns].float().cpu().transpose(-1, -2) / math.sqrt(D)
+    ref_s, _ = oracle.attend(scores, torch.ones(Ns, Ns, dtype=torch.bool).tril(), v[:, :, :Ns].float().cpu())
+    assert_close_16(short.view(B, Ns, H, D).transpose(1, 2).cpu(), ref_s)

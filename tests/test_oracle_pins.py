@@ -252,6 +252,30 @@ def test_quantize_bruteforce_and_first_max_ties():
     assert torch.equal(onehot.argmax(-1), ids) and onehot.sum(-1).eq(1).all()
 
 
+def test_encode_residual_is_stagewise_nearest_neighbour():
+    """Each stage picks the codeword closest (L2, torch.cdist) to the running residual; first minimum on exact ties;
+    the reconstruction error never grows when the codebook holds the zero vector."""
+    B, H, N, M, K, D = 2, 2, 24, 3, 8, 4
+    x = _rand(B, H, N, D, seed=54)
+    cb = _rand(H, M, K, D, seed=55)
+    cb[:, :, 6] = cb[:, :, 1]  # exact duplicate: code 6 must never be chosen
+    cb[:, :, 0] = 0.0
+    codes = oracle.encode_residual(x, cb)
+    assert codes.shape == (B, H, N, M) and not (codes == 6).any()
+    r = x.clone().double()
+    prev = (r * r).sum(-1)
+    for m in range(M):
+        for h in range(H):
+            dist = torch.cdist(r[:, h], cb[h, m].double())  # [B,N,K]
+            assert torch.equal(dist.argmin(-1), codes[:, h, :, m])
+            r[:, h] -= cb[h, m].double()[codes[:, h, :, m]]
+        err = (r * r).sum(-1)
+        assert (err <= prev + 1e-9).all()
+        prev = err
+    # reconstruction through the key-reconstruction oracle leaves exactly that residual
+    torch.testing.assert_close(x.double() - oracle.reconstruct_keys(codes, cb).double(), r, atol=1e-5, rtol=0)
+
+
 def test_preprocess_invariants_bruteforce():
     B, H, N, C, D = 1, 2, 384, 8, 4
     g = torch.Generator().manual_seed(52)

@@ -4,7 +4,7 @@ unimplemented).
 
 Every layer keeps, per (batch, head): the additive-quantiser codes of its keys `[B,H,cap,M] uint8` and the values
 `[B,H,cap,D]`.  A step projects the new token, rotates q to the clamped ReRoPE position, encodes the new key greedily
-against the layer's codebooks (residual, nearest codeword), appends code and value, and attends over the whole cache
+against the layer's codebooks (residual, nearest codeword; HIP encoder), appends code and value, and attends over the whole cache
 with the HIP decode kernel.  The linear layers are plain torch matmuls (weights ~ N(0, 0.02)): they are plumbing around
 the attention path, which is what this harness measures.
 
@@ -18,24 +18,13 @@ import time
 import torch
 
 from .ops.attn_vq import attn_vq_decode, rope_tables, rotate_half
+from .ops.mini_vq import RESIDUAL, encode_keys
 
 
 def encode_residual(x, codebooks):
-    """Greedy additive (residual) encoding: code_m = argmin_c |r - cb[h,m,c]|^2, r -= cb[h,m,code_m].
-
-    x [B,H,T,D], codebooks [H,M,K,D] -> codes [B,H,T,M] uint8.  fp32 arithmetic."""
-    r = x.float()
-    cb = codebooks.float()
-    half_norm = 0.5 * (cb * cb).sum(-1)  # [H,M,K]
-    codes = []
-    for m in range(cb.shape[1]):
-        score = torch.einsum("bhtd,hkd->bhtk", r, cb[:, m]) - half_norm[:, m][None, :, None, :]
-        idx = score.argmax(-1)  # nearest codeword in L2
-        codes.append(idx)
-        picked = cb[:, m].unsqueeze(0).expand(r.shape[0], -1, -1, -1).gather(
-            2, idx.unsqueeze(-1).expand(-1, -1, -1, r.shape[-1]))
-        r = r - picked
-    return torch.stack(codes, dim=-1).to(torch.uint8)
+    """Greedy additive (residual) encoding on the HIP key encoder: x [B,H,T,D], codebooks [H,M,K,D] ->
+    codes [B,H,T,M] uint8."""
+    return encode_keys(x, codebooks, RESIDUAL)[0]
 
 
 class VQDecodeModel:

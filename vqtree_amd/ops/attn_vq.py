@@ -10,7 +10,7 @@ from enum import Enum
 import torch
 
 from .. import _lib
-from .mini_vq import multi_head_single_quantize
+from .mini_vq import multi_head_single_quantize, quantize_ids
 
 BLOCK_SIZE = 128  # granularity of the far-context boundary (ops/attn_vq.py:23)
 
@@ -222,6 +222,39 @@ def sort_based_preprocess(vq_key_ids, vq_key_onehot, value_states, block=BLOCK_S
     return cum[:, :, block - 1::block].contiguous(), v_vq.to(dtype), vi[:, :, block - 1::block].contiguous()
 
 
+def segmented_preprocess(vq_key_ids, value_states, n_codes, block=BLOCK_SIZE, want_int64_counts=False):
+    """Same three tensors as `sort_based_preprocess`, built by the HIP preprocessing kernels (per-block histograms,
+    scan, scatter into (code, position) order, one running fp32 sum per code) instead of the one-hot cumulative sum,
+    argsort and global prefix sum of ops/attn_vq.py:352-384.  Returns (counts [B,H,N//block,C] in the model dtype, or
+    int64 when `want_int64_counts`; v_vq [B,H,N+1,D]; vi [B,H,N//block,C] int64)."""
+    from .. import _lib
+    from ._common import SUFFIX, bhn_strides, ptr
+
+    assert block == BLOCK_SIZE
+    lib = _lib.load()
+    _lib.require_gpu(vq_key_ids, value_states)
+    B, H, N = vq_key_ids.shape
+    D = value_states.shape[-1]
+    dtype, device = value_states.dtype, value_states.device
+    assert dtype in SUFFIX and vq_key_ids.dtype == torch.int64
+    assert n_codes < (1 << 13) and N < (1 << 18), "limits of the reference's sort keys (ops/attn_vq.py:355-359)"
+    value_states = value_states if value_states.stride(-1) == 1 else value_states.contiguous()
+    NT = N // block
+    cnt = torch.empty((B, H, NT, n_codes), dtype=torch.int64 if want_int64_counts else dtype, device=device)
+    vi = torch.empty((B, H, NT, n_codes), dtype=torch.int64, device=device)
+    v_vq = torch.empty((B, H, N + 1, D), dtype=dtype, device=device)
+    ws = torch.empty(lib.vqa_preprocess_workspace_bytes(B, H, N, n_codes), dtype=torch.uint8, device=device)
+    strides = _lib.strides_array(*bhn_strides(vq_key_ids), *bhn_strides(value_states), *bhn_strides(cnt),
+                                 *bhn_strides(cnt), *bhn_strides(v_vq), *bhn_strides(vi))
+    with torch.cuda.device(device):
+        rc = getattr(lib, "vqa_preprocess_" + SUFFIX[dtype])(
+            ptr(vq_key_ids), ptr(value_states), ptr(cnt) if want_int64_counts else None,
+            None if want_int64_counts else ptr(cnt), ptr(v_vq), ptr(vi), ptr(ws), ws.numel(), B, H, N, D, n_codes,
+            strides, _lib.current_stream(device))
+    _lib.check(rc)
+    return cnt, v_vq, vi
+
+
 def long_prefilling_sort_based_linear(query_states, key_states, value_states, position_ids, cache, layer_idx=0,
                                       rope_base=10000.0):
     """Linear-time prefill with VQ memory (ops/attn_vq.py:336-443): encode keys with the head's codebook, build the
@@ -230,10 +263,10 @@ def long_prefilling_sort_based_linear(query_states, key_states, value_states, po
 
     B, H, N, D = query_states.shape
     dtype = query_states.dtype
-    _, ids, onehot = multi_head_single_quantize(key_states, cache.codebook)
-    cnt, v_vq, vi = sort_based_preprocess(ids, onehot, value_states)
+    ids = quantize_ids(key_states, cache.codebook)
+    cnt, v_vq, vi = segmented_preprocess(ids, value_states, cache.codebook.shape[1])
     q1, k1, q2 = rerope_operands(query_states, key_states, position_ids, cache.window_length, rope_base)
-    out = vq_attn_forward(q1, q2, k1, cache.codebook, cnt.to(dtype), key_states, value_states, v_vq, vi,
+    out = vq_attn_forward(q1, q2, k1, cache.codebook, cnt, key_states, value_states, v_vq, vi,
                           cache.window_length, softmax_scale=1 / math.sqrt(D))
     _remember(cache, layer_idx, ids, value_states, N)
     return out.transpose(1, 2).contiguous().flatten(2)
@@ -245,7 +278,7 @@ def long_prefilling_per_key(query_states, key_states, value_states, position_ids
     merge pass.  Needs a codebook of at most 256 entries (uint8 codes)."""
     B, H, N, D = query_states.shape
     assert cache.codebook.shape[1] <= 256
-    _, ids, _ = multi_head_single_quantize(key_states, cache.codebook)
+    ids = quantize_ids(key_states, cache.codebook)
     q1, k1, q2 = rerope_operands(query_states, key_states, position_ids, cache.window_length, rope_base)
     out = attn_vq_prefill(q1, ids.to(torch.uint8).unsqueeze(-1), cache.codebook.unsqueeze(1), value_states,
                           k_exact=k1, window_size=cache.window_length, q2=q2, k2=key_states,
@@ -308,13 +341,13 @@ def dispatch_attn(query_states, key_states, value_states, position_ids, cache, l
         q1, k1, _ = rerope_operands(query_states, key_states, position_ids, cache.window_length, rope_base)
         out = causal_window_attention(q1.transpose(1, 2), k1.transpose(1, 2), value_states.transpose(1, 2), q_len,
                                       softmax_scale=1 / math.sqrt(D))
-        _, ids, _ = multi_head_single_quantize(key_states, cache.codebook)
+        ids = quantize_ids(key_states, cache.codebook)
         _remember(cache, layer_idx, ids, value_states, q_len)
         return out.contiguous().flatten(2)
     assert q_len == 1, "Only support prefilling or generation"
     assert len(cache.key_codes) > layer_idx, "decode needs a codebook of at most 256 entries"
     # generation step: append the new key's code and value, then attend over all codes with the clamped query
-    _, ids, _ = multi_head_single_quantize(key_states, cache.codebook)
+    ids = quantize_ids(key_states, cache.codebook)
     cache.key_codes[layer_idx] = torch.cat([cache.key_codes[layer_idx], ids.to(torch.uint8).unsqueeze(-1)], dim=2)
     cache.value_cache[layer_idx] = torch.cat([cache.value_cache[layer_idx], value_states], dim=2)
     if layer_idx == 0:
