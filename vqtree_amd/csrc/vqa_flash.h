@@ -102,42 +102,51 @@ __device__ __forceinline__ void dma16(const void* gptr, uint32_t lds_addr) {
                  : "memory");  // m0 is written too; no other instruction of these kernels uses it
 }
 
+// same with the global address split into a wave-uniform base (scalar registers) and a 32-bit per-lane byte offset
+__device__ __forceinline__ void dma16_uniform(const void* uniform_base, uint32_t lane_offset, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(lane_offset), "s"(uniform_base), "s"(lds_addr)
+                 : "memory");
+}
+
 __device__ __forceinline__ uint32_t lds_addr_of(const char* p) {
     return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) char*)p;
 }
 
-template <int D, bool kIsV>
+template <int D, bool kIsV, int NW = kWaves>
 struct TileCopy {
+    static constexpr int kRowsPerWave = kBN / NW;                         // rows of the tile one wave brings
+    static constexpr int kInstr = kRowsPerWave / Geom<D>::kRowsPerInstr;  // direct-to-LDS loads per wave and tile
+    static_assert(kInstr >= 1, "too many waves for this tile");
     int wave;
-    int lane_row;                           // row (within the kRowsPerInstr rows of one instruction) of this lane
-    int chunk;                              // LDS chunk column of this lane
-    uint32_t chunk_bytes[Geom<D>::kInstr];  // byte offset inside the global row that lands in that column
+    int lane_row;                  // row (within the kRowsPerInstr rows of one instruction) of this lane
+    int chunk;                     // LDS chunk column of this lane
+    uint32_t chunk_bytes[kInstr];  // byte offset inside the global row that lands in that column
 
     __device__ __forceinline__ void init(int wave_, int lane) {
         wave = wave_;
         lane_row = lane / Geom<D>::kChunksPerRow;
         chunk = lane % Geom<D>::kChunksPerRow;
 #pragma unroll
-        for (int i = 0; i < Geom<D>::kInstr; ++i) chunk_bytes[i] = (uint32_t)src_chunk(row(i)) * 16u;
+        for (int i = 0; i < kInstr; ++i) chunk_bytes[i] = (uint32_t)src_chunk(row(i)) * 16u;
     }
     __device__ __forceinline__ int row(int i) const {
-        return wave * Geom<D>::kRowsPerWave + i * Geom<D>::kRowsPerInstr + lane_row;
+        return wave * kRowsPerWave + i * Geom<D>::kRowsPerInstr + lane_row;
     }
     __device__ __forceinline__ int src_chunk(int r) const {
         return chunk ^ (kIsV ? Geom<D>::swz_v(r) : Geom<D>::swz_k(r));
     }
     __device__ __forceinline__ uint32_t dst(const char* lds_tile, int i) const {
-        return lds_addr_of(lds_tile) + (wave * Geom<D>::kRowsPerWave + i * Geom<D>::kRowsPerInstr) * Geom<D>::kRowBytes;
+        return lds_addr_of(lds_tile) + (wave * kRowsPerWave + i * Geom<D>::kRowsPerInstr) * Geom<D>::kRowBytes;
     }
     // rows [n0, n0+64), all inside the matrix: uniform (scalar) row-group base + one 32-bit per-lane offset
     __device__ __forceinline__ void load_full(const char* lds_tile, const uint16_t* base, int64_t sn, int n0) const {
         const uint32_t lane_off = (uint32_t)lane_row * (uint32_t)(sn * 2);
+        const char* grp = reinterpret_cast<const char*>(base + (int64_t)(n0 + wave * kRowsPerWave) * sn);
+        const int64_t step = (int64_t)Geom<D>::kRowsPerInstr * sn * 2;  // bytes between the row groups of two loads
 #pragma unroll
-        for (int i = 0; i < Geom<D>::kInstr; ++i) {
-            const char* grp = reinterpret_cast<const char*>(
-                base + (int64_t)(n0 + wave * Geom<D>::kRowsPerWave + i * Geom<D>::kRowsPerInstr) * sn);
-            dma16(grp + (lane_off + chunk_bytes[i]), dst(lds_tile, i));
-        }
+        for (int i = 0; i < kInstr; ++i) dma16_uniform(grp + i * step, lane_off + chunk_bytes[i], dst(lds_tile, i));
     }
     // rows [n0, n0+64) of a [n_rows, D] matrix with row stride sn (elements); rows past the end repeat the last row
     __device__ __forceinline__ void load(const char* lds_tile, const uint16_t* base, int64_t sn, int n0,
@@ -146,7 +155,7 @@ struct TileCopy {
             load_full(lds_tile, base, sn, n0);
         } else {
 #pragma unroll
-            for (int i = 0; i < Geom<D>::kInstr; ++i) {
+            for (int i = 0; i < kInstr; ++i) {
                 const int g = min(n0 + row(i), n_rows - 1);
                 const char* src = reinterpret_cast<const char*>(base + (int64_t)g * sn) + chunk_bytes[i];
                 dma16(src, dst(lds_tile, i));
@@ -157,7 +166,7 @@ struct TileCopy {
     __device__ __forceinline__ void load_gather(const char* lds_tile, const uint16_t* base, int64_t sn,
                                                 const int64_t* row_index, int n0, int n_rows) const {
 #pragma unroll
-        for (int i = 0; i < Geom<D>::kInstr; ++i) {
+        for (int i = 0; i < kInstr; ++i) {
             const int64_t g = row_index[min(n0 + row(i), n_rows - 1)];
             const char* src = reinterpret_cast<const char*>(base + g * sn) + chunk_bytes[i];
             dma16(src, dst(lds_tile, i));
@@ -321,6 +330,7 @@ __device__ __forceinline__ void softmax_update(SoftmaxState<D>& st, f32x16_t (&s
         st.m = m_new;
     }
     float sum = 0.f;
+    const uint32_t kOnes = Elem<Tag>::pack2(1.f, 1.f);
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
@@ -331,11 +341,11 @@ __device__ __forceinline__ void softmax_update(SoftmaxState<D>& st, f32x16_t (&s
                 const int r = j2 * 8 + 2 * e;
                 const float p0 = fast_exp2(__builtin_fmaf(s[kb][r], scale, -m_safe));
                 const float p1 = fast_exp2(__builtin_fmaf(s[kb][r + 1], scale, -m_safe));
+                pk[e] = Elem<Tag>::pack2(p0, p1);
                 if constexpr (kWeighted)
                     sum += p0 * w[kb][r] + p1 * w[kb][r + 1];
                 else
-                    sum += p0 + p1;
-                pk[e] = Elem<Tag>::pack2(p0, p1);
+                    sum = Elem<Tag>::dot2(pk[e], kOnes, sum);  // row sum of the ROUNDED pair, as P.V uses it
             }
             p[kb][j2] = __builtin_bit_cast(typename Elem<Tag>::vec8, pk);
         }
