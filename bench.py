@@ -114,6 +114,39 @@ def prefill_extra(dev, steps=20, warmup=5):
     return out
 
 
+def local_rerope_extra(dev, steps=10, warmup=3):
+    """Sliding-window ReRoPE attention at 16k (batch 2, 32 heads, window 512), the exact-window building block of the
+    prefill path: useful FLOPs = 4 * D * visible pairs (keys j <= i with j >= floor(i/128)*128 - window)."""
+    import torch
+
+    from vqtree_amd.ops.attn_vq import rope_tables, rotate_half
+    from vqtree_amd.ops.triton_fused_local_attn_rerope import flash_attn_func
+
+    B, H, N, D, W = 2, 32, 16384, 128, 512
+    g = torch.Generator(device=dev).manual_seed(4)
+    q, k, v = (torch.randn(B, N, H, D, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+               for _ in range(3))
+    cos, sin = rope_tables(D, N, dtype=torch.bfloat16, device=dev)
+    rope = lambda x, c, s_: x * c + rotate_half(x) * s_
+    q1, k1 = rope(q, cos[None, :, None], sin[None, :, None]), rope(k, cos[None, :, None], sin[None, :, None])
+    q2 = rope(q, cos[W + 1], sin[W + 1])
+    ms = _time_events(lambda: flash_attn_func(q1, q2, k1, k, v, W), steps, warmup)
+    i = torch.arange(N, dtype=torch.int64)
+    pairs = int((i - torch.clamp(i // 128 * 128 - W, min=0) + 1).sum())
+    flops = 4 * D * pairs * B * H
+    tf = flops / (ms * 1e-3) / 1e12
+    out = {
+        "workload": f"local ReRoPE window attention: batch {B}, {H} heads, head_dim {D}, seq {N}, window {W}, bf16",
+        "us_per_call": round(ms * 1e3, 1),
+        "useful_gflop": round(flops / 1e9, 1),
+        "tflops": round(tf, 1),
+        "mfma_frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
+    }
+    del q, k, v, q1, k1, q2
+    torch.cuda.empty_cache()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -212,6 +245,7 @@ def main():
         del case
         torch.cuda.empty_cache()
         result["prefill"] = prefill_extra(dev)
+        result["local_rerope"] = local_rerope_extra(dev)
     print(json.dumps(result))
 
 
