@@ -115,3 +115,21 @@ def test_linear_prefill_uses_the_hip_preprocessing_consistently():
     b = A.segmented_preprocess(ids, v, C, want_int64_counts=True)
     assert torch.equal(a[0], b[0]) and torch.equal(a[2], b[2])
     assert_close_16(b[1].cpu(), a[1].cpu(), "v_vq")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,H,N,D", [(2, 3, 257, 128), (1, 2, 100, 64), (1, 1, 7, 16)])
+def test_rotary_kernel_is_bit_exact(dtype, B, H, N, D):
+    """The rotary kernel against the CPU oracle (the expression evaluated operator by operator on 16-bit tensors):
+    bit-exact, for per-row positions, one clamped position, and a strided ([B,N,H,D]-backed) input."""
+    print(f"rope: {dtype} B{B} H{H} N{N} D{D}", flush=True)
+    x = _draw((B, N, H, D), dtype, 13).transpose(1, 2)  # [B,H,N,D] view of a [B,N,H,D] buffer
+    cos, sin = oracle.rope_tables(D, N + 40, dtype=dtype)
+    pos = (torch.arange(N)[None, :] + torch.tensor([[3], [17]])[:B]).contiguous()
+    got = A.apply_rope(x.cuda(), cos.cuda(), sin.cuda(), pos.cuda()).cpu()
+    for b in range(B):
+        want = oracle.apply_rope(x[b], cos, sin, pos[b])
+        assert torch.equal(got[b], want)
+    got_fixed = A.apply_rope(x.cuda(), cos.cuda(), sin.cuda(), 33).cpu()
+    assert torch.equal(got_fixed, oracle.apply_rope(x, cos, sin, 33))
+    assert torch.equal(A.apply_rope(x.cuda(), cos.cuda(), sin.cuda(), 0).cpu(), x)  # position 0 is the identity

@@ -6,7 +6,7 @@ import math
 
 import torch
 
-from .attn_vq import rope_tables, rotate_half
+from .attn_vq import apply_rope, rope_tables, rotate_half
 from .triton_fused_attn_rerope import attention
 from .triton_fused_local_attn import flash_attn_func as causal_window_attention
 
@@ -65,11 +65,7 @@ class ReRoPECache:
 
 def _rope_at(x, cos, sin, positions):
     """x [B,H,N,D]; positions: LongTensor [B,N] or a single int."""
-    if isinstance(positions, int):
-        c, s = cos[positions], sin[positions]
-    else:
-        c, s = cos[positions].unsqueeze(1), sin[positions].unsqueeze(1)
-    return x * c + rotate_half(x) * s
+    return apply_rope(x, cos, sin, positions)
 
 
 def rerope_attn_forward(query_states, key_states, value_states, position_ids, cache, layer_idx=0, rope_base=10000.0):

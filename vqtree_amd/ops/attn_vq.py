@@ -185,17 +185,52 @@ def rope_tables(head_dim, n_pos, base=10000.0, dtype=torch.float32, device=None)
     return emb.cos().to(dtype), emb.sin().to(dtype)
 
 
+def apply_rope(x, cos, sin, positions):
+    """x * cos[p] + rotate_half(x) * sin[p] for x [B,H,N,D]; `positions` is a LongTensor [B,N] or one int for every
+    row.  16-bit tensors on the GPU run the HIP rotary kernel, whose rounding (each product and the sum rounded to the
+    element type) is that of this very expression evaluated on 16-bit tensors; anything else evaluates the expression
+    with torch operators."""
+    from .. import _lib
+    from ._common import SUFFIX, bhn_strides, ptr
+
+    if x.is_cuda and x.dtype in SUFFIX and cos.dtype == x.dtype and x.shape[-1] % 16 == 0:
+        lib = _lib.load()
+        B, H, N, D = x.shape
+        x = x if x.stride(-1) == 1 else x.contiguous()
+        cos = cos if cos.stride(-1) == 1 else cos.contiguous()
+        sin = sin if sin.stride(-1) == 1 and sin.stride(0) == cos.stride(0) else sin.contiguous()
+        if sin.stride(0) != cos.stride(0):
+            cos = cos.contiguous()
+        out = torch.empty((B, H, N, D), dtype=x.dtype, device=x.device)
+        fixed = isinstance(positions, int)
+        if not fixed:
+            positions = positions.to(torch.int64)
+            assert positions.shape == (B, N)
+        strides = _lib.strides_array(*bhn_strides(x), *((0, 0) if fixed else (positions.stride(0), positions.stride(1))),
+                                     *bhn_strides(out))
+        with torch.cuda.device(x.device):
+            rc = getattr(lib, "vqa_rope_" + SUFFIX[x.dtype])(ptr(x), None if fixed else ptr(positions), ptr(cos),
+                                                             ptr(sin), ptr(out), B, H, N, D, cos.shape[0],
+                                                             cos.stride(0), strides, positions if fixed else 0,
+                                                             _lib.current_stream(x.device))
+        _lib.check(rc)
+        return out
+    if isinstance(positions, int):
+        c, s = cos[positions], sin[positions]
+    else:
+        c, s = cos[positions].unsqueeze(1), sin[positions].unsqueeze(1)  # [B,1,N,D]
+    return x * c + rotate_half(x) * s
+
+
 def rerope_operands(query_states, key_states, position_ids, window_length, rope_base=10000.0):
     """(q1, k1, q2) of ops/attn_vq.py:402-407: rotary at the true positions, and the query at the clamped position
     window_length + 1.  position_ids [B,N]; states [B,H,N,D]."""
     B, H, N, D = query_states.shape
     n_pos = max(int(position_ids.max()) + 1, window_length + 2)
     cos, sin = rope_tables(D, n_pos, rope_base, query_states.dtype, query_states.device)
-    c, s = cos[position_ids].unsqueeze(1), sin[position_ids].unsqueeze(1)  # [B,1,N,D]
-    q1 = query_states * c + rotate_half(query_states) * s
-    k1 = key_states * c + rotate_half(key_states) * s
-    cw, sw = cos[window_length + 1], sin[window_length + 1]
-    q2 = query_states * cw + rotate_half(query_states) * sw
+    q1 = apply_rope(query_states, cos, sin, position_ids)
+    k1 = apply_rope(key_states, cos, sin, position_ids)
+    q2 = apply_rope(query_states, cos, sin, window_length + 1)
     return q1, k1, q2
 
 
