@@ -179,6 +179,18 @@ int vqa_vqcount_fwd_f16(const void* q2, const void* k_vq, const void* k_vq_cnt, 
                         void* out, float* lse, int B, int H, int N, int D, int C, const int64_t* strides, int window,
                         float sm_scale, vqa_stream_t stream);
 
+/* Same kernel with the merge fused into its epilogue: out [B,H,N,D] / lse [B,H,N] (contiguous) already hold an
+ * attention state (the window kernel's o1, l1) and receive merge((o1, l1), (o2, l2)) in place; rows below window + 128
+ * are left untouched.  Replaces the count kernel launch plus the flashinfer merge and its four layout copies
+ * (ops/triton_fused_vq_attn.py:222-250) by one launch. */
+int vqa_vqcount_merge_bf16(const void* q2, const void* k_vq, const void* k_vq_cnt, const void* v_vq, const int64_t* vi,
+                           void* out, float* lse, int B, int H, int N, int D, int C, const int64_t* strides,
+                           int window, float sm_scale, vqa_stream_t stream);
+
+int vqa_vqcount_merge_f16(const void* q2, const void* k_vq, const void* k_vq_cnt, const void* v_vq, const int64_t* vi,
+                          void* out, float* lse, int B, int H, int N, int D, int C, const int64_t* strides, int window,
+                          float sm_scale, vqa_stream_t stream);
+
 /* ------------------------------------------------------------------------------------------------------------------
  * In-place merge of two attention states with base-2 log-sum-exp: m = max(s, s'), o <- (o 2^(s-m) + o' 2^(s'-m)) /
  * (2^(s-m) + 2^(s'-m)), s <- m + log2(2^(s-m) + 2^(s'-m)); a side with s = -inf is ignored.

@@ -30,6 +30,8 @@ SIGNATURES = {
     "vqa_prefill_f32": (c_int, [_P] * 6 + [c_int] * 6 + [_STRIDES, c_int, c_float, _P]),
     "vqa_vqcount_fwd_bf16": (c_int, [_P] * 7 + [c_int] * 5 + [_STRIDES, c_int, c_float, _P]),
     "vqa_vqcount_fwd_f16": (c_int, [_P] * 7 + [c_int] * 5 + [_STRIDES, c_int, c_float, _P]),
+    "vqa_vqcount_merge_bf16": (c_int, [_P] * 7 + [c_int] * 5 + [_STRIDES, c_int, c_float, _P]),
+    "vqa_vqcount_merge_f16": (c_int, [_P] * 7 + [c_int] * 5 + [_STRIDES, c_int, c_float, _P]),
     "vqa_merge_state_inplace_bf16": (c_int, [_P] * 4 + [c_int] * 4 + [_STRIDES, _P]),
     "vqa_merge_state_inplace_f16": (c_int, [_P] * 4 + [c_int] * 4 + [_STRIDES, _P]),
     "vqa_encode_keys_bf16": (c_int, [_P] * 4 + [c_int] * 6 + [_STRIDES, c_int, c_int, _P]),

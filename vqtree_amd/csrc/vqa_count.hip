@@ -21,6 +21,7 @@ struct CountParams {
     int64_t o_sb, o_sh, o_sn;
     float* lse;             // [B,H,N]
     int H, N, C, window, n_far_tiles;
+    int merge_into;  // out / lse already hold an attention state: merge this kernel's state into it
     float scale_log2e;
 };
 
@@ -28,9 +29,12 @@ template <typename Tag, int D>
 __global__ __launch_bounds__(kThreads, 2) void count_kernel(CountParams p) {
     typedef Geom<D> G;
     typedef typename Elem<Tag>::vec8 vec8;
-    __shared__ __attribute__((aligned(1024))) char s_k[G::kTileBytes];
-    __shared__ __attribute__((aligned(1024))) char s_v[G::kTileBytes];
-    __shared__ float s_cnt[kBN];
+    // dynamic LDS (4 tiles + 2 x 64 counts is 512 bytes past the 64 KB static limit at D = 128):
+    // K tiles | V tiles | counts, each double-buffered
+    extern __shared__ __attribute__((aligned(1024))) char smem[];
+    char(*s_k)[G::kTileBytes] = reinterpret_cast<char(*)[G::kTileBytes]>(smem);
+    char(*s_v)[G::kTileBytes] = reinterpret_cast<char(*)[G::kTileBytes]>(smem + 2 * G::kTileBytes);
+    float(*s_cnt)[kBN] = reinterpret_cast<float(*)[kBN]>(smem + 4 * G::kTileBytes);
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -72,40 +76,96 @@ __global__ __launch_bounds__(kThreads, 2) void count_kernel(CountParams p) {
     k_copy.init(wave, lane);
     v_copy.init(wave, lane);
 
-    for (int c0 = 0; c0 < p.C; c0 += kBN) {
-        float cnt_f = 0.f;
-        if (tid < kBN && c0 + tid < p.C) cnt_f = Elem<Tag>::from_bits(cnt[c0 + tid]);
-        __syncthreads();  // previous tile fully consumed
-        k_copy.load(s_k, cb, p.cb_sc, c0, p.C);
-        v_copy.load_gather(s_v, vvq, p.vvq.sn, vi, c0, p.C);
-        if (tid < kBN) s_cnt[tid] = cnt_f;  // 0 for codewords past C: masked below
+    // codeword tiles are double-buffered: tile c+1 (codebook rows, gathered V sums, counts) is requested before
+    // tile c is computed
+    auto request = [&](int c0, int buf) {
+        k_copy.load(s_k[buf], cb, p.cb_sc, c0, p.C);
+        v_copy.load_gather(s_v[buf], vvq, p.vvq.sn, vi, c0, p.C);
+        if (tid < kBN) s_cnt[buf][tid] = (c0 + tid < p.C) ? Elem<Tag>::from_bits(cnt[c0 + tid]) : 0.f;  // 0: masked
+    };
+    request(0, 0);
+    int buf = 0;
+    for (int c0 = 0; c0 < p.C; c0 += kBN, buf ^= 1) {
         wait_tile_loads();
-        __syncthreads();
+        __syncthreads();  // tile c0 is complete in `buf`; every wave is done with the other buffer
+        if (c0 + kBN < p.C) request(c0 + kBN, buf ^ 1);
 
         f32x16_t s[2];
-        qk_mma<Tag, D>(s, q, s_k, lane);
+        qk_mma<Tag, D>(s, q, s_k[buf], lane);
         float w[2][16];
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const float c = s_cnt[kb * 32 + key_of_reg(r, half)];
+                const float c = s_cnt[buf][kb * 32 + key_of_reg(r, half)];
                 w[kb][r] = c;
                 s[kb][r] = (c != 0.f) ? s[kb][r] : -INFINITY;
             }
         vec8 pf[2][2];
         softmax_update<Tag, D, true>(st, s, p.scale_log2e, pf, w);
-        pv_mma<Tag, D>(st.o, pf, s_v, lane);
+        pv_mma<Tag, D>(st.o, pf, s_v[buf], lane);
     }
-    store_output<Tag, D>(st, out_base, p.o_sn, lse_base, row0, p.N, lane);
+    if (!p.merge_into) {
+        store_output<Tag, D>(st, out_base, p.o_sn, lse_base, row0, p.N, lane);
+        return;
+    }
+    // merge with the state already in out / lse (base-2 log-sum-exp), in place
+    {
+        const int n = lane & 31;
+        const int row = row0 + n;
+        if (row >= p.N) return;
+        const float l_tot = st.l + __shfl_xor(st.l, 32, 64);
+        const float s2 = l_tot > 0.f ? st.m + fast_log2(l_tot) : -INFINITY;
+        const float s1 = lse_base[row];
+        const float mx = fmaxf(s1, s2);
+        const float m_safe = (mx == -INFINITY) ? 0.f : mx;
+        const float w1 = fast_exp2(s1 - m_safe), w2 = fast_exp2(s2 - m_safe);
+        const float den = w1 + w2;
+        const float inv = den > 0.f ? 1.f / den : 0.f;
+        const float f1 = w1 * inv;                                  // weight of the stored (normalised) output
+        const float f2 = l_tot > 0.f ? w2 * inv / l_tot : 0.f;      // weight of this kernel's unnormalised sums
+        uint16_t* dst = out_base + (int64_t)row * p.o_sn;
+#pragma unroll
+        for (int db = 0; db < Geom<D>::kDBlocks; ++db) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                uint2* at = reinterpret_cast<uint2*>(dst + db * 32 + 8 * g + 4 * half);
+                const uint2 old = *at;
+                const uint32_t ow[2] = {old.x, old.y};
+                uint32_t nw[2];
+#pragma unroll
+                for (int e = 0; e < 2; ++e) {
+                    const float lo = Elem<Tag>::from_bits((uint16_t)(ow[e] & 0xffffu)) * f1 + st.o[db][4 * g + 2 * e] * f2;
+                    const float hi = Elem<Tag>::from_bits((uint16_t)(ow[e] >> 16)) * f1 + st.o[db][4 * g + 2 * e + 1] * f2;
+                    nw[e] = (uint32_t)Elem<Tag>::to_bits(lo) | ((uint32_t)Elem<Tag>::to_bits(hi) << 16);
+                }
+                *at = make_uint2(nw[0], nw[1]);
+            }
+        }
+        if (half == 0) lse_base[row] = den > 0.f ? mx + fast_log2(den) : -INFINITY;
+    }
+}
+
+template <typename Tag, int D>
+int launch_count(const CountParams& p, dim3 grid, hipStream_t stream) {
+    constexpr size_t kLds = 4 * Geom<D>::kTileBytes + 2 * kBN * sizeof(float);
+    if (kLds > 65536 &&
+        hipFuncSetAttribute(reinterpret_cast<const void*>(&count_kernel<Tag, D>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLds) != hipSuccess) {
+        (void)hipGetLastError();
+        return VQA_ERR_LAUNCH_FAILED;
+    }
+    hipLaunchKernelGGL((count_kernel<Tag, D>), grid, dim3(kThreads), kLds, stream, p);
+    return launch_status();
 }
 
 // strides: q2(b,h,n) k_vq(h,c) k_vq_cnt(b,h,t) v_vq(b,h,n) vi(b,h,t) out(b,h,n)
 template <typename Tag>
 int vqcount(const void* q2, const void* k_vq, const void* k_vq_cnt, const void* v_vq, const int64_t* vi, void* out,
             float* lse, int B, int H, int N, int D, int C, const int64_t* strides, int window, float sm_scale,
-            hipStream_t stream) {
+            bool merge_into, hipStream_t stream) {
     if (!q2 || !k_vq || !k_vq_cnt || !v_vq || !vi || !out || !strides) return VQA_ERR_NULL_POINTER;
+    if (merge_into && !lse) return VQA_ERR_NULL_POINTER;
     if (B <= 0 || H <= 0 || N <= 0 || C <= 0) return VQA_ERR_BAD_SHAPE;
     if (window < 0 || !(sm_scale > 0.f) || (int64_t)B * H > 65535) return VQA_ERR_BAD_ARGUMENT;
     CountParams p;
@@ -129,15 +189,15 @@ int vqcount(const void* q2, const void* k_vq, const void* k_vq_cnt, const void* 
         return VQA_ERR_MISALIGNED;
     const int first = window + kTile;
     p.n_far_tiles = N > first ? (N - first + kTile - 1) / kTile : 0;
-    const int zero_tiles = ((first < N ? first : N) + kBM - 1) / kBM;
+    p.merge_into = merge_into ? 1 : 0;
+    // rows below window + 128 have no far context: zero / -inf when this kernel writes a state of its own, left
+    // untouched when it merges into an existing one
+    const int zero_tiles = merge_into ? 0 : ((first < N ? first : N) + kBM - 1) / kBM;
+    if (p.n_far_tiles + zero_tiles == 0) return VQA_OK;
     const dim3 grid(p.n_far_tiles + zero_tiles, B * H);
-    if (D == 64)
-        hipLaunchKernelGGL((count_kernel<Tag, 64>), grid, dim3(kThreads), 0, stream, p);
-    else if (D == 128)
-        hipLaunchKernelGGL((count_kernel<Tag, 128>), grid, dim3(kThreads), 0, stream, p);
-    else
-        return VQA_ERR_UNSUPPORTED_HEAD_DIM;
-    return launch_status();
+    if (D == 64) return launch_count<Tag, 64>(p, grid, stream);
+    if (D == 128) return launch_count<Tag, 128>(p, grid, stream);
+    return VQA_ERR_UNSUPPORTED_HEAD_DIM;
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -230,14 +290,28 @@ int vqa_vqcount_fwd_bf16(const void* q2, const void* k_vq, const void* k_vq_cnt,
                          void* out, float* lse, int B, int H, int N, int D, int C, const int64_t* strides, int window,
                          float sm_scale, vqa_stream_t stream) {
     return vqa::flash::vqcount<vqa::bf16_tag>(q2, k_vq, k_vq_cnt, v_vq, vi, out, lse, B, H, N, D, C, strides, window,
-                                              sm_scale, stream);
+                                              sm_scale, false, stream);
 }
 
 int vqa_vqcount_fwd_f16(const void* q2, const void* k_vq, const void* k_vq_cnt, const void* v_vq, const int64_t* vi,
                         void* out, float* lse, int B, int H, int N, int D, int C, const int64_t* strides, int window,
                         float sm_scale, vqa_stream_t stream) {
     return vqa::flash::vqcount<vqa::f16_tag>(q2, k_vq, k_vq_cnt, v_vq, vi, out, lse, B, H, N, D, C, strides, window,
-                                             sm_scale, stream);
+                                             sm_scale, false, stream);
+}
+
+int vqa_vqcount_merge_bf16(const void* q2, const void* k_vq, const void* k_vq_cnt, const void* v_vq, const int64_t* vi,
+                           void* out, float* lse, int B, int H, int N, int D, int C, const int64_t* strides,
+                           int window, float sm_scale, vqa_stream_t stream) {
+    return vqa::flash::vqcount<vqa::bf16_tag>(q2, k_vq, k_vq_cnt, v_vq, vi, out, lse, B, H, N, D, C, strides, window,
+                                              sm_scale, true, stream);
+}
+
+int vqa_vqcount_merge_f16(const void* q2, const void* k_vq, const void* k_vq_cnt, const void* v_vq, const int64_t* vi,
+                          void* out, float* lse, int B, int H, int N, int D, int C, const int64_t* strides, int window,
+                          float sm_scale, vqa_stream_t stream) {
+    return vqa::flash::vqcount<vqa::f16_tag>(q2, k_vq, k_vq_cnt, v_vq, vi, out, lse, B, H, N, D, C, strides, window,
+                                             sm_scale, true, stream);
 }
 
 int vqa_merge_state_inplace_bf16(void* o, float* s, const void* o_other, const float* s_other, int B, int H, int N,

@@ -25,11 +25,9 @@ def merge_state_in_place(v, s, v_other, s_other):
     return v, s
 
 
-def vq_count_forward(q2, k_vq, k_vq_cnt, v_vq, vi, window_size, softmax_scale=None):
-    """Far-context kernel alone: (o2 [B,H,N,D], lse2 [B,H,N] fp32 base 2); rows i < window+128 are 0 / -inf."""
+def _count_call(q2, k_vq, k_vq_cnt, v_vq, vi, window_size, softmax_scale, out, lse, merge):
     lib = _lib.load()
     _lib.require_gpu(q2, k_vq, k_vq_cnt, v_vq, vi)
-    q2, k_vq, k_vq_cnt, v_vq, vi = last_dim_contiguous(q2, k_vq, k_vq_cnt, v_vq, vi)
     B, H, N, D = q2.shape
     C = k_vq.shape[1]
     sfx = check_same_16bit(q2, k_vq, k_vq_cnt, v_vq)
@@ -37,16 +35,23 @@ def vq_count_forward(q2, k_vq, k_vq_cnt, v_vq, vi, window_size, softmax_scale=No
     assert k_vq_cnt.shape[-1] == C and vi.shape == k_vq_cnt.shape
     n_far = max(0, -(-(N - window_size - 128) // 128))
     assert k_vq_cnt.shape[2] >= n_far, "k_vq_cnt / vi need one row per far-context query tile"
+    strides = _lib.strides_array(*bhn_strides(q2), k_vq.stride(0), k_vq.stride(1), *bhn_strides(k_vq_cnt),
+                                 *bhn_strides(v_vq), *bhn_strides(vi), *bhn_strides(out))
+    with torch.cuda.device(q2.device):
+        rc = getattr(lib, ("vqa_vqcount_merge_" if merge else "vqa_vqcount_fwd_") + sfx)(
+            ptr(q2), ptr(k_vq), ptr(k_vq_cnt), ptr(v_vq), ptr(vi), ptr(out), ptr(lse), B, H, N, D, C, strides,
+            int(window_size), softmax_scale, _lib.current_stream(q2.device))
+    _lib.check(rc)
+
+
+def vq_count_forward(q2, k_vq, k_vq_cnt, v_vq, vi, window_size, softmax_scale=None):
+    """Far-context kernel alone: (o2 [B,H,N,D], lse2 [B,H,N] fp32 base 2); rows i < window+128 are 0 / -inf."""
+    q2, k_vq, k_vq_cnt, v_vq, vi = last_dim_contiguous(q2, k_vq, k_vq_cnt, v_vq, vi)
+    B, H, N, D = q2.shape
     softmax_scale = softmax_scale or 1.0 / math.sqrt(D)
     o2 = torch.empty((B, H, N, D), dtype=q2.dtype, device=q2.device)
     l2 = torch.empty((B, H, N), dtype=torch.float32, device=q2.device)
-    strides = _lib.strides_array(*bhn_strides(q2), k_vq.stride(0), k_vq.stride(1), *bhn_strides(k_vq_cnt),
-                                 *bhn_strides(v_vq), *bhn_strides(vi), *bhn_strides(o2))
-    with torch.cuda.device(q2.device):
-        rc = getattr(lib, "vqa_vqcount_fwd_" + sfx)(ptr(q2), ptr(k_vq), ptr(k_vq_cnt), ptr(v_vq), ptr(vi), ptr(o2),
-                                                    ptr(l2), B, H, N, D, C, strides, int(window_size), softmax_scale,
-                                                    _lib.current_stream(q2.device))
-    _lib.check(rc)
+    _count_call(q2, k_vq, k_vq_cnt, v_vq, vi, window_size, softmax_scale, o2, l2, merge=False)
     return o2, l2
 
 
@@ -55,19 +60,13 @@ def vq_attn_forward(q1, q2, k1, k_vq, k_vq_cnt, k3, v, v_vq, vi, window_size, so
     [B,H,N//128,C] running counts / prefix-sum row indices sampled per 128-key block; k3 raw keys; v_vq [B,H,N+1,D]
     per-code prefix sums of V.  All attention tensors [B,H,N,D].  Returns [B,H,N,D].
 
-    Unlike the reference (batch == 1 only, four layout copies around the merge) the three kernels work on the
-    [B,H,N,D] tensors in place and any batch size is accepted.
+    Unlike the reference (batch == 1 only, four layout copies around a separate merge launch) the two kernels work on
+    the [B,H,N,D] tensors in place, the merge is the count kernel's epilogue, and any batch size is accepted.
     """
     q1, q2, k1, k_vq, k_vq_cnt, k3, v, v_vq, vi = last_dim_contiguous(q1, q2, k1, k_vq, k_vq_cnt, k3, v, v_vq, vi)
-    lib = _lib.load()
     B, H, N, D = q1.shape
     softmax_scale = softmax_scale or 1.0 / math.sqrt(D)
     o1, l1 = local_attention_bhnd(q1, q2, k1, k3, v, window_size, LOCAL_REROPE, softmax_scale, True)
-    o2, l2 = vq_count_forward(q2, k_vq, k_vq_cnt, v_vq, vi, window_size, softmax_scale)
-    sfx = check_same_16bit(o1, o2)
-    strides = _lib.strides_array(*bhn_strides(o1), *bhn_strides(l1), *bhn_strides(o2), *bhn_strides(l2))
-    with torch.cuda.device(q1.device):
-        rc = getattr(lib, "vqa_merge_state_inplace_" + sfx)(ptr(o1), ptr(l1), ptr(o2), ptr(l2), B, H, N, D, strides,
-                                                            _lib.current_stream(q1.device))
-    _lib.check(rc)
+    # far context, merged into (o1, l1) by the count kernel's epilogue
+    _count_call(q2, k_vq, k_vq_cnt, v_vq, vi, window_size, softmax_scale, o1, l1, merge=True)
     return o1
