@@ -6,7 +6,8 @@
 //   v_vq[0]    = 0;   v_vq[1 + r] = sum of V over the keys of r's code up to and including sorted row r,
 //                where keys are ordered by (code, position)
 //
-// Four passes per (batch, head): per-128-key histograms; a running sum over blocks plus an exclusive scan over codes;
+// Passes per (batch, head): per-128-key histograms; a running sum over blocks, an exclusive scan over codes and the
+// block-sampled outputs;
 // a scatter of key positions into sorted order (rank = start + keys of the code in earlier blocks + earlier keys of
 // the code in the same block); one wave per code walking its segment with an fp32 running sum.
 #include "vqa_common.h"
@@ -54,28 +55,30 @@ __global__ __launch_bounds__(kBlock) void hist_kernel(Params p) {
     for (int c = threadIdx.x; c < p.C; c += kBlock) out[c] = s_hist[c];
 }
 
-template <typename Tag>
-__global__ __launch_bounds__(256) void scan_kernel(Params p) {
-    __shared__ int s_total[kMaxCodes];
+// running count over blocks, in place; one thread per code.  total[c] lands in `start` until start_kernel replaces it.
+__global__ __launch_bounds__(256) void cumulate_kernel(Params p) {
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    const int bh = blockIdx.y;
+    if (c >= p.C) return;
+    int32_t* hist = p.hist + (int64_t)bh * p.NB * p.C + c;
+    int run = 0;
+    for (int t = 0; t < p.NB; ++t) {
+        run += hist[(int64_t)t * p.C];
+        hist[(int64_t)t * p.C] = run;
+    }
+    p.start[(int64_t)bh * p.C + c] = run;
+}
+
+// start[c] = exclusive prefix sum of the totals over codes; one workgroup per (batch, head)
+__global__ __launch_bounds__(256) void start_kernel(Params p) {
     __shared__ int s_part[256];
     const int bh = blockIdx.x;
-    const int b = bh / p.H, h = bh % p.H;
     const int tid = threadIdx.x;
-    int32_t* hist = p.hist + (int64_t)bh * p.NB * p.C;
-    for (int c = tid; c < p.C; c += 256) {
-        int run = 0;
-        for (int t = 0; t < p.NB; ++t) {
-            run += hist[(int64_t)t * p.C + c];
-            hist[(int64_t)t * p.C + c] = run;
-        }
-        s_total[c] = run;
-    }
-    __syncthreads();
-    // exclusive scan over codes: every thread owns a contiguous strip
-    const int strip = (p.C + 255) / 256;
+    int32_t* start = p.start + (int64_t)bh * p.C;
+    const int strip = (p.C + 255) / 256;  // every thread owns a contiguous strip of codes
     const int c_lo = min(tid * strip, p.C), c_hi = min(c_lo + strip, p.C);
     int sum = 0;
-    for (int c = c_lo; c < c_hi; ++c) sum += s_total[c];
+    for (int c = c_lo; c < c_hi; ++c) sum += start[c];
     s_part[tid] = sum;
     __syncthreads();
     if (tid == 0) {
@@ -89,22 +92,23 @@ __global__ __launch_bounds__(256) void scan_kernel(Params p) {
     __syncthreads();
     int run = s_part[tid];
     for (int c = c_lo; c < c_hi; ++c) {
-        const int x = s_total[c];
-        s_total[c] = run;
+        const int x = start[c];
+        start[c] = run;
         run += x;
     }
-    __syncthreads();
-    int32_t* start = p.start + (int64_t)bh * p.C;
-    for (int c = tid; c < p.C; c += 256) start[c] = s_total[c];
-    const int NT = p.N / kBlock;
-    for (int t = 0; t < NT; ++t) {
-        for (int c = tid; c < p.C; c += 256) {
-            const int n = hist[(int64_t)t * p.C + c];
-            if (p.cnt) p.cnt[b * p.cn_sb + h * p.cn_sh + (int64_t)t * p.cn_st + c] = n;
-            if (p.cnt_elem) p.cnt_elem[b * p.ce_sb + h * p.ce_sh + (int64_t)t * p.ce_st + c] = Elem<Tag>::to_bits((float)n);
-            p.vi[b * p.vi_sb + h * p.vi_sh + (int64_t)t * p.vi_st + c] = (int64_t)n + s_total[c];
-        }
-    }
+}
+
+// block-sampled outputs: cnt[t, c], its element-type copy, vi[t, c] = cnt + start[c]
+template <typename Tag>
+__global__ __launch_bounds__(256) void emit_kernel(Params p) {
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    const int t = blockIdx.y, bh = blockIdx.z;
+    const int b = bh / p.H, h = bh % p.H;
+    if (c >= p.C) return;
+    const int n = p.hist[((int64_t)bh * p.NB + t) * p.C + c];
+    if (p.cnt) p.cnt[b * p.cn_sb + h * p.cn_sh + (int64_t)t * p.cn_st + c] = n;
+    if (p.cnt_elem) p.cnt_elem[b * p.ce_sb + h * p.ce_sh + (int64_t)t * p.ce_st + c] = Elem<Tag>::to_bits((float)n);
+    p.vi[b * p.vi_sb + h * p.vi_sh + (int64_t)t * p.vi_st + c] = (int64_t)n + p.start[(int64_t)bh * p.C + c];
 }
 
 __global__ __launch_bounds__(kBlock) void scatter_kernel(Params p) {
@@ -123,6 +127,8 @@ __global__ __launch_bounds__(kBlock) void scatter_kernel(Params p) {
     p.order[(int64_t)bh * p.N + rank] = j;
 }
 
+// One wave per code: running fp32 sum of V over the code's keys in position order.  The sorted positions are
+// fetched 64 at a time (one per lane) and the V rows eight at a time, so only the additions form a dependent chain.
 template <typename Tag>
 __global__ __launch_bounds__(256) void segment_sum_kernel(Params p) {
     const int lane = threadIdx.x & 63;
@@ -132,21 +138,34 @@ __global__ __launch_bounds__(256) void segment_sum_kernel(Params p) {
     if (c >= p.C) return;
     const int d = lane * 2;
     const bool live = d < p.D;
-    uint16_t* out = p.vvq + b * p.vq_sb + h * p.vq_sh + d;
+    const int dd = live ? d : 0;  // idle lanes shadow column 0 and never store
+    uint16_t* out = p.vvq + b * p.vq_sb + h * p.vq_sh + dd;
     if (c == 0 && live) *reinterpret_cast<uint32_t*>(out) = 0u;  // row 0
     const int s = p.start[(int64_t)bh * p.C + c];
     const int e = s + p.hist[((int64_t)bh * p.NB + p.NB - 1) * p.C + c];
     const int32_t* order = p.order + (int64_t)bh * p.N;
-    const uint16_t* v = p.v + b * p.v_sb + h * p.v_sh + d;
+    const uint16_t* v = p.v + b * p.v_sb + h * p.v_sh + dd;
     float a0 = 0.f, a1 = 0.f;
-    for (int r = s; r < e; ++r) {
-        const int j = order[r];
-        if (live) {
-            const uint32_t w = *reinterpret_cast<const uint32_t*>(v + (int64_t)j * p.v_sn);
-            a0 += Elem<Tag>::from_bits((uint16_t)(w & 0xffffu));
-            a1 += Elem<Tag>::from_bits((uint16_t)(w >> 16));
-            *reinterpret_cast<uint32_t*>(out + (int64_t)(1 + r) * p.vq_sn) =
-                (uint32_t)Elem<Tag>::to_bits(a0) | ((uint32_t)Elem<Tag>::to_bits(a1) << 16);
+    for (int r0 = s; r0 < e; r0 += 64) {
+        const int n = min(64, e - r0);
+        const int mine = order[r0 + min(lane, n - 1)];
+        for (int k0 = 0; k0 < n; k0 += 8) {
+            uint32_t w[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int j = __shfl(mine, min(k0 + u, n - 1), 64);
+                w[u] = *reinterpret_cast<const uint32_t*>(v + (int64_t)j * p.v_sn);
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                if (k0 + u < n) {
+                    a0 += Elem<Tag>::from_bits((uint16_t)(w[u] & 0xffffu));
+                    a1 += Elem<Tag>::from_bits((uint16_t)(w[u] >> 16));
+                    if (live)
+                        *reinterpret_cast<uint32_t*>(out + (int64_t)(1 + r0 + k0 + u) * p.vq_sn) =
+                            (uint32_t)Elem<Tag>::to_bits(a0) | ((uint32_t)Elem<Tag>::to_bits(a1) << 16);
+                }
+            }
         }
     }
 }
@@ -166,7 +185,7 @@ int preprocess(const int64_t* ids, const void* v, int64_t* cnt, void* cnt_elem, 
                hipStream_t stream) {
     if (!ids || !v || !v_vq || !workspace || !strides) return VQA_ERR_NULL_POINTER;
     if (!vi && N >= kBlock) return VQA_ERR_NULL_POINTER;  // no block-sampled row exists below 128 keys
-    if (B <= 0 || H <= 0 || N <= 0 || C <= 0 || C > kMaxCodes || N > (1 << 24)) return VQA_ERR_BAD_SHAPE;
+    if (B <= 0 || H <= 0 || N <= 0 || C <= 0 || C > kMaxCodes || N / kBlock > 65535) return VQA_ERR_BAD_SHAPE;
     if (D < 2 || D > 128 || (D & 1)) return VQA_ERR_UNSUPPORTED_HEAD_DIM;
     if ((int64_t)B * H > 65535) return VQA_ERR_BAD_ARGUMENT;
     if (ws_bytes < workspace_bytes(B, H, N, C)) return VQA_ERR_WORKSPACE_TOO_SMALL;
@@ -196,7 +215,10 @@ int preprocess(const int64_t* ids, const void* v, int64_t* cnt, void* cnt_elem, 
     ws += align256(bh * C * 4);
     p.order = reinterpret_cast<int32_t*>(ws);
     hipLaunchKernelGGL(hist_kernel, dim3(p.NB, B * H), dim3(kBlock), C * sizeof(int), stream, p);
-    hipLaunchKernelGGL((scan_kernel<Tag>), dim3(B * H), dim3(256), 0, stream, p);
+    hipLaunchKernelGGL(cumulate_kernel, dim3((C + 255) / 256, B * H), dim3(256), 0, stream, p);
+    hipLaunchKernelGGL(start_kernel, dim3(B * H), dim3(256), 0, stream, p);
+    if (N / kBlock > 0)
+        hipLaunchKernelGGL((emit_kernel<Tag>), dim3((C + 255) / 256, N / kBlock, B * H), dim3(256), 0, stream, p);
     hipLaunchKernelGGL(scatter_kernel, dim3(p.NB, B * H), dim3(kBlock), 0, stream, p);
     hipLaunchKernelGGL((segment_sum_kernel<Tag>), dim3((C + 3) / 4, B * H), dim3(256), 0, stream, p);
     return launch_status();

@@ -176,13 +176,23 @@ def rotate_half(x):
     return torch.cat((-x[..., half:], x[..., :half]), dim=-1)
 
 
+_ROPE_TABLE_CACHE = {}
+
+
 def rope_tables(head_dim, n_pos, base=10000.0, dtype=torch.float32, device=None):
     """cos / sin [n_pos, D] of the transformers ~4.37 rotary embedding the reference's modules call
-    (inv_freq = base^(-2r/D), emb = cat(freqs, freqs)), cast to the model dtype."""
-    inv_freq = 1.0 / (base ** (torch.arange(0, head_dim, 2, dtype=torch.float32, device=device) / head_dim))
-    freqs = torch.outer(torch.arange(n_pos, dtype=torch.float32, device=device), inv_freq)
-    emb = torch.cat((freqs, freqs), dim=-1)
-    return emb.cos().to(dtype), emb.sin().to(dtype)
+    (inv_freq = base^(-2r/D), emb = cat(freqs, freqs)), cast to the model dtype.  Tables are kept per
+    (head_dim, base, dtype, device) and grown in powers of two, like the model's own cached rotary module."""
+    key = (head_dim, float(base), dtype, str(device))
+    have = _ROPE_TABLE_CACHE.get(key)
+    if have is None or have[0].shape[0] < n_pos:
+        size = 1 << max(0, int(n_pos) - 1).bit_length()
+        inv_freq = 1.0 / (base ** (torch.arange(0, head_dim, 2, dtype=torch.float32, device=device) / head_dim))
+        freqs = torch.outer(torch.arange(size, dtype=torch.float32, device=device), inv_freq)
+        emb = torch.cat((freqs, freqs), dim=-1)
+        have = (emb.cos().to(dtype), emb.sin().to(dtype))
+        _ROPE_TABLE_CACHE[key] = have
+    return have[0][:n_pos], have[1][:n_pos]
 
 
 def apply_rope(x, cos, sin, positions):
