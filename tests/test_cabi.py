@@ -75,3 +75,38 @@ def test_ops_refuse_cpu_tensors():
     with pytest.raises(_lib.VqaError):
         attn_vq_decode(q, torch.zeros(1, 1, 8, 4, dtype=torch.uint8), torch.zeros(1, 4, 256, 128, dtype=torch.bfloat16),
                        torch.zeros(1, 1, 8, 128, dtype=torch.bfloat16))
+
+
+def test_encoder_preprocessing_rope_reject_bad_arguments_before_any_launch(lib):
+    s12, s18, s8 = (_lib.strides_array(*([8] * n)) for n in (12, 18, 8))
+    enc = lambda x=16, cb=16, codes=16, ids=None, N=8, D=128, M=4, K=256, mode=1: lib.vqa_encode_keys_bf16(
+        x, cb, codes, ids, 1, 1, N, D, M, K, s12, mode, 0, None)
+    assert enc(x=None) == -1 and enc(codes=None, ids=None) == -1   # VQA_ERR_NULL_POINTER
+    assert enc(N=0) == -2 and enc(K=250) == -2                      # VQA_ERR_BAD_SHAPE (K must be a multiple of 32)
+    assert enc(D=96) == -3                                          # VQA_ERR_UNSUPPORTED_HEAD_DIM
+    assert enc(K=512) == -7 and enc(mode=2) == -7                   # uint8 codes need K <= 256; unknown mode
+    assert enc(x=18) == -5                                          # VQA_ERR_MISALIGNED
+
+    need = lib.vqa_preprocess_workspace_bytes(2, 4, 1000, 512)
+    # histograms [B*H, ceil(N/128), C] + start [B*H, C] + order [B*H, N], int32 each
+    assert need >= 8 * 8 * 512 * 4 + 8 * 512 * 4 + 8 * 1000 * 4 and need % 256 == 0
+    assert lib.vqa_preprocess_workspace_bytes(0, 4, 1000, 512) == 0
+    pre = lambda ids=16, v=16, vvq=16, vi=16, ws=256, ws_bytes=1 << 30, N=1000, D=128, C=512: lib.vqa_preprocess_bf16(
+        ids, v, None, None, vvq, vi, ws, ws_bytes, 2, 4, N, D, C, s18, None)
+    assert pre(ids=None) == -1 and pre(vi=None) == -1
+    assert pre(C=8193) == -2 and pre(N=0) == -2
+    assert pre(D=130) == -3 and pre(D=7) == -3
+    assert pre(ws_bytes=need - 1) == -6                             # VQA_ERR_WORKSPACE_TOO_SMALL
+    assert pre(ws=128) == -5
+
+    rope = lambda x=16, pos=16, cos=16, sin=16, out=16, D=128, n_pos=64, fixed=0: lib.vqa_rope_bf16(
+        x, pos, cos, sin, out, 1, 1, 8, D, n_pos, 128, s8, fixed, None)
+    assert rope(x=None) == -1 and rope(cos=None) == -1
+    assert rope(D=24) == -3
+    assert rope(pos=None, fixed=64) == -7 and rope(pos=None, fixed=-1) == -7   # fixed position outside the tables
+    assert rope(out=20) == -5
+
+    s17 = _lib.strides_array(*([8] * 17))
+    merge = lambda lse=16, out=16: lib.vqa_vqcount_merge_bf16(16, 16, 16, 16, 16, out, lse, 1, 1, 256, 128, 128, s17,
+                                                              64, 1.0, None)
+    assert merge(lse=None) == -1 and merge(out=None) == -1          # the state to merge into is required
