@@ -241,7 +241,7 @@ def test_count_kernel_and_merge_separately():
 @pytest.mark.parametrize("B,H,N,D,M,K,causal", [(1, 8, 1024, 64, 2, 256, True), (2, 2, 333, 128, 4, 256, True),
                                                  (1, 2, 1500, 64, 1, 100, False), (1, 1, 70, 128, 8, 256, True)])
 def test_vq_prefill_fp32_config1(B, H, N, D, M, K, causal):
-    """BASELINE configuration 1 (batch 1, 8 heads, 1024 tokens, head_dim 64, fp32, 2 x 256 codebooks ~N(0, 0.5)) and
+    """Validation configuration 1 (batch 1, 8 heads, 1024 tokens, head_dim 64, fp32, 2 x 256 codebooks ~N(0, 0.5)) and
     variations, against the naive softmax(Q K_hat^T / sqrt(d)) V to 1e-4."""
     _say(f"vq prefill fp32 B{B} H{H} N{N} D{D} M{M} K{K} causal={causal}")
     g = torch.Generator("cpu").manual_seed(1)
