@@ -76,19 +76,31 @@ __global__ __launch_bounds__(kThreads, 2) void count_kernel(CountParams p) {
     k_copy.init(wave, lane);
     v_copy.init(wave, lane);
 
-    // codeword tiles are double-buffered: tile c+1 (codebook rows, gathered V sums, counts) is requested before
-    // tile c is computed
-    auto request = [&](int c0, int buf) {
-        k_copy.load(s_k[buf], cb, p.cb_sc, c0, p.C);
-        v_copy.load_gather(s_v[buf], vvq, p.vvq.sn, vi, c0, p.C);
-        if (tid < kBN) s_cnt[buf][tid] = (c0 + tid < p.C) ? Elem<Tag>::from_bits(cnt[c0 + tid]) : 0.f;  // 0: masked
+    // Codeword tiles are double-buffered: tile c+1 (codebook rows, gathered V sums, counts) is requested before tile
+    // c is computed.  The row indices and counts of a tile are fetched into registers one tile earlier still, so the
+    // request never waits on them.
+    int64_t rows[TileCopy<D, true>::kInstr];
+    float cnt_f = 0.f;
+    auto fetch_meta = [&](int c0) {
+        v_copy.fetch_rows(rows, vi, c0, p.C);
+        cnt_f = (tid < kBN && c0 + tid < p.C) ? Elem<Tag>::from_bits(cnt[c0 + tid]) : 0.f;  // 0: masked
     };
+    auto request = [&](int c0, int buf) {  // uses the metadata fetched for c0
+        k_copy.load(s_k[buf], cb, p.cb_sc, c0, p.C);
+        v_copy.load_rows(s_v[buf], vvq, p.vvq.sn, rows);
+        if (tid < kBN) s_cnt[buf][tid] = cnt_f;
+    };
+    fetch_meta(0);
     request(0, 0);
+    if (kBN < p.C) fetch_meta(kBN);
     int buf = 0;
     for (int c0 = 0; c0 < p.C; c0 += kBN, buf ^= 1) {
         wait_tile_loads();
         __syncthreads();  // tile c0 is complete in `buf`; every wave is done with the other buffer
-        if (c0 + kBN < p.C) request(c0 + kBN, buf ^ 1);
+        if (c0 + kBN < p.C) {
+            request(c0 + kBN, buf ^ 1);
+            if (c0 + 2 * kBN < p.C) fetch_meta(c0 + 2 * kBN);
+        }
 
         f32x16_t s[2];
         qk_mma<Tag, D>(s, q, s_k[buf], lane);
@@ -96,10 +108,14 @@ __global__ __launch_bounds__(kThreads, 2) void count_kernel(CountParams p) {
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const float c = s_cnt[buf][kb * 32 + key_of_reg(r, half)];
-                w[kb][r] = c;
-                s[kb][r] = (c != 0.f) ? s[kb][r] : -INFINITY;
+            for (int g = 0; g < 4; ++g) {
+                // registers 4g .. 4g+3 hold codewords kb*32 + 8g + 4*half + 0..3: one 16-byte LDS read
+                const f32x4_t c4 = *reinterpret_cast<const f32x4_t*>(&s_cnt[buf][kb * 32 + 8 * g + 4 * half]);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    w[kb][4 * g + e] = c4[e];
+                    s[kb][4 * g + e] = (c4[e] != 0.f) ? s[kb][4 * g + e] : -INFINITY;
+                }
             }
         vec8 pf[2][2];
         softmax_update<Tag, D, true>(st, s, p.scale_log2e, pf, w);

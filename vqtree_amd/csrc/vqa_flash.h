@@ -162,13 +162,18 @@ struct TileCopy {
             }
         }
     }
-    // same with the global row taken from an index list
-    __device__ __forceinline__ void load_gather(const char* lds_tile, const uint16_t* base, int64_t sn,
-                                                const int64_t* row_index, int n0, int n_rows) const {
+    // same with the global rows taken from an index list, in two steps so that the indices can be fetched a tile
+    // ahead of the copy that uses them: rows[i] = row_index[n0 + row(i)] (clamped), then one copy per index
+    __device__ __forceinline__ void fetch_rows(int64_t (&rows)[kInstr], const int64_t* row_index, int n0,
+                                               int n_rows) const {
+#pragma unroll
+        for (int i = 0; i < kInstr; ++i) rows[i] = row_index[min(n0 + row(i), n_rows - 1)];
+    }
+    __device__ __forceinline__ void load_rows(const char* lds_tile, const uint16_t* base, int64_t sn,
+                                              const int64_t (&rows)[kInstr]) const {
 #pragma unroll
         for (int i = 0; i < kInstr; ++i) {
-            const int64_t g = row_index[min(n0 + row(i), n_rows - 1)];
-            const char* src = reinterpret_cast<const char*>(base + g * sn) + chunk_bytes[i];
+            const char* src = reinterpret_cast<const char*>(base + rows[i] * sn) + chunk_bytes[i];
             dma16(src, dst(lds_tile, i));
         }
     }

@@ -1,0 +1,61 @@
+"""Timing of the reference-shaped long-prefill route (single codebook per head, count-weighted far context) and of its
+stages, next to the fused per-key formulation, at the prefill benchmark shape.
+
+    python -m vqtree_amd.route_bench [--heads 32 --tokens 8192 --window 1024 --codes 512]
+
+Prints one JSON object; times are medians of HIP-event intervals in microseconds."""
+import argparse
+import json
+
+import torch
+
+from .ops import attn_vq as A
+from .ops import mini_vq as Q
+from .ops.triton_fused_vq_attn import vq_attn_forward
+
+
+def _time(fn, steps=10, warmup=3):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    for s, e in ev:
+        s.record()
+        fn()
+        e.record()
+    torch.cuda.synchronize()
+    t = sorted(s.elapsed_time(e) for s, e in ev)
+    return round(t[len(t) // 2] * 1e3, 1)
+
+
+def run(batch=1, heads=32, tokens=8192, head_dim=128, window=1024, codes=512, device="cuda"):
+    B, H, N, D, W, C = batch, heads, tokens, head_dim, window, codes
+    g = torch.Generator(device=device).manual_seed(1)
+    q, k, v = (torch.randn(B, H, N, D, generator=g, device=device).bfloat16() for _ in range(3))
+    cb = torch.randn(H, C, D, generator=g, device=device).bfloat16()
+    pos = torch.arange(N, device=device).unsqueeze(0).expand(B, -1)
+    q1, k1, q2 = A.rerope_operands(q, k, pos, W)
+    ids = Q.quantize_ids(k, cb)
+    cnt, v_vq, vi = A.segmented_preprocess(ids, v, C)
+    out = {
+        "workload": f"long prefill with VQ memory: batch {B}, {H} heads, {N} tokens, head_dim {D}, window {W}, "
+                    f"{C} codewords per head, bf16",
+        "encode_keys_us": _time(lambda: Q.quantize_ids(k, cb)),
+        "preprocess_us": _time(lambda: A.segmented_preprocess(ids, v, C)),
+        "rotary_operands_us": _time(lambda: A.rerope_operands(q, k, pos, W)),
+        "vq_attn_forward_us": _time(lambda: vq_attn_forward(q1, q2, k1, cb, cnt, k, v, v_vq, vi, W)),
+        "dispatch_attn_whole_us": _time(lambda: A.dispatch_attn(q, k, v, pos, A.VectorQuantizedReRoPECache(W, cb))),
+    }
+    # the same attention through the fused per-key kernel (needs uint8 codes: at most 256 codewords)
+    cb256 = cb[:, :256].contiguous()
+    ids256 = Q.quantize_ids(k, cb256).to(torch.uint8).unsqueeze(-1)
+    out["fused_per_key_256_codewords_us"] = _time(
+        lambda: A.attn_vq_prefill(q1, ids256, cb256.unsqueeze(1), v, k_exact=k1, window_size=W, q2=q2, k2=k))
+    return out
+
+
+if __name__ == "__main__":
+    ap = argparse.ArgumentParser()
+    for name, default in (("batch", 1), ("heads", 32), ("tokens", 8192), ("window", 1024), ("codes", 512)):
+        ap.add_argument("--" + name, type=int, default=default)
+    print(json.dumps(run(**vars(ap.parse_args()))))
