@@ -108,14 +108,6 @@ __device__ __forceinline__ float score_from_lut(const float* s_lut, typename Cod
     }
 }
 
-// 16-byte load of data that is read exactly once (V rows): the non-temporal hint keeps the stream from displacing
-// the lines that are re-read; measured on a 4 GiB read-only sweep it lifts the rate from ~6.3 to ~7.1 TB/s.
-typedef uint32_t stream_u32x4_t __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ uint4 load_stream16(const char* p) {
-    const stream_u32x4_t t = __builtin_nontemporal_load(reinterpret_cast<const stream_u32x4_t*>(p));
-    return make_uint4(t[0], t[1], t[2], t[3]);
-}
-
 // Lane layout inside a wave: LPR = D/8 lanes cover one V row with 16-byte loads, so one load instruction covers
 // G = 64/LPR consecutive rows; a 64-key batch takes R = 64/G loads per lane.  Lane (g, c) accumulates rows
 // {i*G + g} into its 8 output elements c*8..c*8+7; the G row groups are summed once at the end.

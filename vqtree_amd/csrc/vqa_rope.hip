@@ -44,7 +44,7 @@ __global__ __launch_bounds__(256) void rope_kernel(Params p) {
     const uint16_t* cr = p.cos + pos * p.t_sp;
     const uint16_t* sr = p.sin + pos * p.t_sp;
     uint16_t* orow = p.out + b * p.o_sb + h * p.o_sh + (int64_t)n * p.o_sn;
-    const uint4 xl = *reinterpret_cast<const uint4*>(xr + c), xh = *reinterpret_cast<const uint4*>(xr + half_d + c);
+    const uint4 xl = load_stream16(xr + c), xh = load_stream16(xr + half_d + c);
     const uint4 cl = *reinterpret_cast<const uint4*>(cr + c), ch = *reinterpret_cast<const uint4*>(cr + half_d + c);
     const uint4 sl = *reinterpret_cast<const uint4*>(sr + c), sh = *reinterpret_cast<const uint4*>(sr + half_d + c);
     const uint32_t xlw[4] = {xl.x, xl.y, xl.z, xl.w}, xhw[4] = {xh.x, xh.y, xh.z, xh.w};
@@ -69,8 +69,8 @@ __global__ __launch_bounds__(256) void rope_kernel(Params p) {
         olw[e] = lo_pair;
         ohw[e] = hi_pair;
     }
-    *reinterpret_cast<uint4*>(orow + c) = make_uint4(olw[0], olw[1], olw[2], olw[3]);
-    *reinterpret_cast<uint4*>(orow + half_d + c) = make_uint4(ohw[0], ohw[1], ohw[2], ohw[3]);
+    store_stream16(orow + c, make_uint4(olw[0], olw[1], olw[2], olw[3]));
+    store_stream16(orow + half_d + c, make_uint4(ohw[0], ohw[1], ohw[2], ohw[3]));
 }
 
 // strides: x(b,h,n) position_ids(b,n) out(b,h,n); the tables are [n_pos, D] with row stride table_stride
