@@ -208,6 +208,27 @@ int vqa_merge_state_inplace_f16(void* o, float* s, const void* o_other, const fl
                                 int D, const int64_t* strides, vqa_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------------------------------
+ * seqlen_q = 1 attention over exact keys: out[b,h] = softmax_j(sm_scale * <q[b,h], k[b,h,j]>) . v[b,h,j], no mask.
+ * The generation step of the ReRoPE module and the short-context fallback of the VQ module make this call through a
+ * third-party flash-attention package in the reference (ops/attn_rerope.py:279-286, ops/attn_vq.py:463-477); with
+ * lse it also yields the exact-window state that vqa_merge_state_inplace combines with vqa_decode's far-context state.
+ *
+ *   q, out [B,H,1,D]; k, v [B,H,N,D]; lse [B,H] (nullable); D in {64,128}.
+ *   strides[0..9] = q(b,h) k(b,h,n) v(b,h,n) out(b,h).  Workspace: vqa_decode_exact_workspace_bytes, 256-byte aligned.
+ * ------------------------------------------------------------------------------------------------------------------ */
+#define VQA_DECODE_EXACT_NUM_STRIDES 10
+
+size_t vqa_decode_exact_workspace_bytes(int B, int H, int N, int D, int num_splits);
+
+int vqa_decode_exact_bf16(const void* q, const void* k, const void* v, void* out, float* lse, void* workspace,
+                          size_t workspace_bytes, int B, int H, int N, int D, const int64_t* strides, float sm_scale,
+                          int num_splits, vqa_stream_t stream);
+
+int vqa_decode_exact_f16(const void* q, const void* k, const void* v, void* out, float* lse, void* workspace,
+                         size_t workspace_bytes, int B, int H, int N, int D, const int64_t* strides, float sm_scale,
+                         int num_splits, vqa_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------------------------------
  * Key encoder: nearest-codeword search of every key against its head's codebooks.
  *   mode 0: id_m = argmax_c <x, codebooks[h,m,c]> for every codebook m independently (inner product, first maximum
  *           on ties) -- replaces multi_head_single_quantize, ops/mini_vq.py:4-18 (M = 1); with round_scores != 0 the

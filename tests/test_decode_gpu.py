@@ -104,3 +104,44 @@ def test_full_size_sampled_units():
                                                case.codebooks[h:h + 1], case.v[b:b + 1, h:h + 1], case.softmax_scale)
         assert_close_16(out[b:b + 1, h:h + 1], want, f"unit {b},{h}")
         assert_close_lse(lse[b:b + 1, h:h + 1], want_lse)
+
+
+# ------------------------------------------------------------------ exact-key decode
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,H,N,D", [(2, 3, 1000, 128), (1, 2, 1, 128), (1, 1, 63, 64), (2, 2, 64, 128), (1, 2, 65, 64),
+                                     (1, 4, 4097, 128), (3, 1, 300, 64)])
+def test_exact_decode_matches_dense_softmax(dtype, B, H, N, D):
+    from vqtree_amd.ops.attn_vq import attn_exact_decode
+
+    print(f"exact decode: {dtype} B{B} H{H} N{N} D{D}", flush=True)
+    g = torch.Generator("cpu").manual_seed(21)
+    q = torch.randn(B, H, 1, D, generator=g).to(dtype)
+    k = torch.randn(B, N, H, D, generator=g).to(dtype).transpose(1, 2)  # strided [B,H,N,D] view
+    v = torch.randn(B, H, N, D, generator=g).to(dtype)
+    scale = 1.0 / math.sqrt(D)
+    want, want_lse = oracle.attend(q.float() @ k.float().transpose(-1, -2) * scale,
+                                   torch.ones(1, N, dtype=torch.bool), v.float())
+    out, lse = attn_exact_decode(q.cuda(), k.cuda(), v.cuda(), return_lse=True)
+    assert_close_16(out.cpu(), want, "exact decode")
+    assert_close_lse(lse.cpu()[..., 0], want_lse[..., 0])
+    for splits in (1, 3, 7):
+        o2 = attn_exact_decode(q.cuda(), k.cuda(), v.cuda(), num_splits=splits)
+        assert_close_16(o2.cpu(), want, f"exact decode, {splits} splits")
+
+
+def test_hybrid_decode_state_merge():
+    """Far keys through their codes, the last `W` keys exactly, merged by log-sum-exp: equals dense attention over
+    [reconstructed far keys ; exact window keys]."""
+    from vqtree_amd.ops.attn_vq import attn_vq_decode_windowed
+
+    B, H, N, D, M, W = 2, 4, 900, 128, 4, 200
+    case = decode_case(B, H, N, D, M, device="cuda", seed=22)
+    g = torch.Generator("cpu").manual_seed(23)
+    k_win = torch.randn(B, H, W, D, generator=g).bfloat16().cuda()
+    far = N - W
+    merged = attn_vq_decode_windowed(case.q, case.codes, case.codebooks, case.v, k_win)
+    k_hat = oracle.reconstruct_keys(case.codes[:, :, :far].cpu(), case.codebooks.cpu())
+    keys = torch.cat([k_hat, k_win.float().cpu()], dim=2)
+    scores = case.q.float().cpu() @ keys.transpose(-1, -2) * case.softmax_scale
+    want, _ = oracle.attend(scores, torch.ones(1, N, dtype=torch.bool), case.v.float().cpu())
+    assert_close_16(merged.cpu(), want, "hybrid decode")

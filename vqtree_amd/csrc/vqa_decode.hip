@@ -302,6 +302,182 @@ __global__ __launch_bounds__(D) void merge_kernel(const float* __restrict__ part
     if (lse != nullptr && d == 0) lse[bh] = l > 0.f ? m_all + fast_log2(l) : -INFINITY;
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// Exact-key variant of the streaming kernel: score_j = sm_scale * <q, K_j> from the key rows themselves (no codes, no
+// lookup table).  Same lane layout for K as for V (LPR lanes per row, G rows per load, R loads per 64-key batch): a
+// lane multiplies its 8-element slice of the row with its slice of q, the LPR lanes of the row add up, and every lane
+// of row group g ends up holding the R scores of its own rows -- exactly the weights it needs for its V rows, so no
+// exchange through LDS is needed.  Both row-buffer sets roll as in the coded kernel.  HBM bound: 2 rows per key.
+// ---------------------------------------------------------------------------------------------------------------
+struct ExactStrides {
+    int64_t q_b, q_h;
+    int64_t k_b, k_h, k_n;
+    int64_t v_b, v_h, v_n;
+};
+
+template <typename Tag, int D>
+__global__ __launch_bounds__(kThreads, 2) void exact_kernel(const uint16_t* __restrict__ q,
+                                                            const uint16_t* __restrict__ k,
+                                                            const uint16_t* __restrict__ v,
+                                                            float* __restrict__ part_o, float* __restrict__ part_ml,
+                                                            int H, int N, int S, int keys_per_split, ExactStrides st,
+                                                            float scale_log2e) {
+    constexpr int LPR = D / 8;
+    constexpr int G = kWave / LPR;
+    constexpr int R = kBatch / G;
+    constexpr int kStep = kWaves * kBatch;
+
+    __shared__ float s_red[kWaves][G][D];
+    __shared__ float s_m[kWaves];
+    __shared__ float s_l[kWaves];
+
+    const int split = blockIdx.x;
+    const int bh = blockIdx.y;
+    const int b = bh / H, h = bh % H;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int g = lane / LPR, c = lane % LPR;
+
+    const uint4 qv = *reinterpret_cast<const uint4*>(q + b * st.q_b + h * st.q_h + c * 8);
+    const uint32_t qw[4] = {qv.x, qv.y, qv.z, qv.w};
+
+    const int k_begin = split * keys_per_split;
+    const int k_end = min(N, k_begin + keys_per_split);
+    const char* k_bh = reinterpret_cast<const char*>(k + b * st.k_b + h * st.k_h);
+    const char* v_bh = reinterpret_cast<const char*>(v + b * st.v_b + h * st.v_h);
+    const int64_t k_row_bytes = st.k_n * 2, v_row_bytes = st.v_n * 2;
+    const uint32_t k_lane_off = (uint32_t)(g * k_row_bytes) + c * 16, k_grp = (uint32_t)(G * k_row_bytes);
+    const uint32_t v_lane_off = (uint32_t)(g * v_row_bytes) + c * 16, v_grp = (uint32_t)(G * v_row_bytes);
+
+    float m_run = -INFINITY;
+    float l_run = 0.f;  // sum over this lane's row group only; the groups are added at the end
+    float acc[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+    uint4 kbuf[R], vbuf[R];
+
+    const int k0 = k_begin + wave * kBatch;
+    const int n_batches = k0 < k_end ? (k_end - k0 + kStep - 1) / kStep : 0;
+    auto batch_bounds = [&](int j, int& load_from, int& valid_from) {
+        valid_from = k0 + j * kStep;
+        load_from = (valid_from + kBatch <= k_end) ? valid_from : max(k_end - kBatch, 0);
+    };
+
+    auto process = [&](auto prefetch, int load_from, int valid_from, int next_load_from) {
+        constexpr bool kPrefetch = decltype(prefetch)::value;
+        const char* next_k = k_bh + (int64_t)next_load_from * k_row_bytes;
+        const char* next_v = v_bh + (int64_t)next_load_from * v_row_bytes;
+        float sc[R];
+        float m_loc = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < R; ++i) {
+            const uint32_t w[4] = {kbuf[i].x, kbuf[i].y, kbuf[i].z, kbuf[i].w};
+            float part = 0.f;
+#pragma unroll
+            for (int d = 0; d < 4; ++d) part = Elem<Tag>::dot2(w[d], qw[d], part);
+#pragma unroll
+            for (int off = LPR / 2; off > 0; off >>= 1) part += __shfl_xor(part, off, 64);
+            const int key = load_from + i * G + g;
+            sc[i] = (key >= valid_from && key < k_end) ? part * scale_log2e : -INFINITY;
+            m_loc = fmaxf(m_loc, sc[i]);
+            if constexpr (kPrefetch) {
+                kbuf[i] = load_stream16(next_k + (k_lane_off + i * k_grp));
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+#pragma unroll
+        for (int off = LPR; off < kWave; off <<= 1) m_loc = fmaxf(m_loc, __shfl_xor(m_loc, off, 64));
+        const float m_new = fmaxf(m_run, m_loc);
+        if (m_new > m_run) {  // same outcome in every lane of the wave
+            const float alpha = fast_exp2(m_run - m_new);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[e] *= alpha;
+            l_run *= alpha;
+            m_run = m_new;
+        }
+#pragma unroll
+        for (int i = 0; i < R; ++i) {
+            float p = (sc[i] == -INFINITY) ? 0.f : fast_exp2(sc[i] - m_run);
+            p = Elem<Tag>::round_keep_f32(p);  // P is rounded to the V type before P.V; l sums the same values
+            l_run += p;
+            const uint32_t pbits = Elem<Tag>::rounded_to_bits(p);
+            const uint32_t p_lo = pbits, p_hi = pbits << 16;
+            const uint32_t w[4] = {vbuf[i].x, vbuf[i].y, vbuf[i].z, vbuf[i].w};
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                acc[2 * d] = Elem<Tag>::dot2(w[d], p_lo, acc[2 * d]);
+                acc[2 * d + 1] = Elem<Tag>::dot2(w[d], p_hi, acc[2 * d + 1]);
+            }
+            if constexpr (kPrefetch) {
+                vbuf[i] = load_stream16(next_v + (v_lane_off + i * v_grp));
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    };
+
+    if (n_batches > 0) {
+        int load_from, valid_from;
+        batch_bounds(0, load_from, valid_from);
+        if (N >= kBatch) {
+            const char* kb = k_bh + (int64_t)load_from * k_row_bytes;
+            const char* vb = v_bh + (int64_t)load_from * v_row_bytes;
+#pragma unroll
+            for (int i = 0; i < R; ++i) kbuf[i] = load_stream16(kb + (k_lane_off + i * k_grp));
+#pragma unroll
+            for (int i = 0; i < R; ++i) vbuf[i] = load_stream16(vb + (v_lane_off + i * v_grp));
+        } else {  // fewer keys than one batch in the whole sequence: clamp rows (their weight is zero)
+#pragma unroll
+            for (int i = 0; i < R; ++i) {
+                const int64_t row = min(i * G + g, N - 1);
+                kbuf[i] = load_stream16(k_bh + row * k_row_bytes + c * 16);
+                vbuf[i] = load_stream16(v_bh + row * v_row_bytes + c * 16);
+            }
+        }
+        for (int j = 0; j + 1 < n_batches; ++j) {
+            int next_load_from, next_valid_from;
+            batch_bounds(j + 1, next_load_from, next_valid_from);
+            process(std::true_type{}, load_from, valid_from, next_load_from);
+            load_from = next_load_from;
+            valid_from = next_valid_from;
+        }
+        process(std::false_type{}, load_from, valid_from, load_from);
+    }
+
+    // combine the G row groups of each wave and the waves of the workgroup
+    float l_wave = l_run;
+#pragma unroll
+    for (int off = LPR; off < kWave; off <<= 1) l_wave += __shfl_xor(l_wave, off, 64);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) s_red[wave][g][c * 8 + e] = acc[e];
+    if (lane == 0) {
+        s_m[wave] = m_run;
+        s_l[wave] = l_wave;
+    }
+    __syncthreads();
+    if (tid < D) {
+        float m_all = s_m[0];
+#pragma unroll
+        for (int w = 1; w < kWaves; ++w) m_all = fmaxf(m_all, s_m[w]);
+        float o = 0.f, l = 0.f;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) {
+            const float wgt = (s_m[w] == -INFINITY) ? 0.f : fast_exp2(s_m[w] - m_all);
+            float t = 0.f;
+#pragma unroll
+            for (int gg = 0; gg < G; ++gg) t += s_red[w][gg][tid];
+            o += wgt * t;
+            l += wgt * s_l[w];
+        }
+        const int64_t slot = (int64_t)bh * S + split;
+        part_o[slot * D + tid] = o;
+        if (tid == 0) {
+            part_ml[slot * 2] = m_all;
+            part_ml[slot * 2 + 1] = l;
+        }
+    }
+}
+
 inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
 struct Workspace {
@@ -400,10 +576,76 @@ int run(const void* q, const uint8_t* codes, const void* codebooks, const void* 
     return run_d<Tag, 128>(q, codes, codebooks, v, out, lse, workspace, B, H, N, M, K, st, sm_scale, S, stream);
 }
 
+// strides: q(b,h) k(b,h,n) v(b,h,n) out(b,h)
+template <typename Tag>
+int run_exact(const void* q, const void* k, const void* v, void* out, float* lse, void* workspace,
+              size_t workspace_bytes, int B, int H, int N, int D, const int64_t* strides, float sm_scale,
+              int num_splits, hipStream_t stream) {
+    if (!q || !k || !v || !out || !workspace || !strides) return VQA_ERR_NULL_POINTER;
+    if (B <= 0 || H <= 0 || N <= 0) return VQA_ERR_BAD_SHAPE;
+    if (D != 64 && D != 128) return VQA_ERR_UNSUPPORTED_HEAD_DIM;
+    ExactStrides es;
+    es.q_b = strides[0], es.q_h = strides[1];
+    es.k_b = strides[2], es.k_h = strides[3], es.k_n = strides[4];
+    es.v_b = strides[5], es.v_h = strides[6], es.v_n = strides[7];
+    Strides st = {};
+    st.o_b = strides[8], st.o_h = strides[9];
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || ((uintptr_t)workspace & 255u)) return VQA_ERR_MISALIGNED;
+    if ((es.q_b | es.q_h | es.k_b | es.k_h | es.k_n | es.v_b | es.v_h | es.v_n) & 7) return VQA_ERR_MISALIGNED;
+    const int S = num_splits > 0 ? num_splits : default_splits(B, H, N);
+    if (S > 65535 || (int64_t)B * H > 65535) return VQA_ERR_BAD_ARGUMENT;
+    const Workspace ws = plan(B, H, D, 0, S);
+    if (workspace_bytes < ws.total) return VQA_ERR_WORKSPACE_TOO_SMALL;
+    char* base = static_cast<char*>(workspace);
+    float* po = reinterpret_cast<float*>(base + ws.po_off);
+    float* pml = reinterpret_cast<float*>(base + ws.pml_off);
+    int kps = (N + S - 1) / S;
+    kps = (kps + kThreads - 1) / kThreads * kThreads;
+    const uint16_t* q16 = static_cast<const uint16_t*>(q);
+    const uint16_t* k16 = static_cast<const uint16_t*>(k);
+    const uint16_t* v16 = static_cast<const uint16_t*>(v);
+    if (D == 64) {
+        hipLaunchKernelGGL((exact_kernel<Tag, 64>), dim3(S, B * H), dim3(kThreads), 0, stream, q16, k16, v16, po, pml,
+                           H, N, S, kps, es, sm_scale * kLog2e);
+    } else {
+        hipLaunchKernelGGL((exact_kernel<Tag, 128>), dim3(S, B * H), dim3(kThreads), 0, stream, q16, k16, v16, po, pml,
+                           H, N, S, kps, es, sm_scale * kLog2e);
+    }
+    int rc = launch_status();
+    if (rc != VQA_OK) return rc;
+    if (D == 64)
+        hipLaunchKernelGGL((merge_kernel<Tag, 64>), dim3(B * H), dim3(64), 0, stream, po, pml,
+                           static_cast<uint16_t*>(out), lse, H, S, st);
+    else
+        hipLaunchKernelGGL((merge_kernel<Tag, 128>), dim3(B * H), dim3(128), 0, stream, po, pml,
+                           static_cast<uint16_t*>(out), lse, H, S, st);
+    return launch_status();
+}
+
 }  // namespace decode
 }  // namespace vqa
 
 extern "C" {
+
+size_t vqa_decode_exact_workspace_bytes(int B, int H, int N, int D, int num_splits) {
+    if (B <= 0 || H <= 0 || N <= 0 || D <= 0) return 0;
+    const int S = num_splits > 0 ? num_splits : vqa::decode::default_splits(B, H, N);
+    return vqa::decode::plan(B, H, D, 0, S).total;
+}
+
+int vqa_decode_exact_bf16(const void* q, const void* k, const void* v, void* out, float* lse, void* workspace,
+                          size_t workspace_bytes, int B, int H, int N, int D, const int64_t* strides, float sm_scale,
+                          int num_splits, vqa_stream_t stream) {
+    return vqa::decode::run_exact<vqa::bf16_tag>(q, k, v, out, lse, workspace, workspace_bytes, B, H, N, D, strides,
+                                                 sm_scale, num_splits, stream);
+}
+
+int vqa_decode_exact_f16(const void* q, const void* k, const void* v, void* out, float* lse, void* workspace,
+                         size_t workspace_bytes, int B, int H, int N, int D, const int64_t* strides, float sm_scale,
+                         int num_splits, vqa_stream_t stream) {
+    return vqa::decode::run_exact<vqa::f16_tag>(q, k, v, out, lse, workspace, workspace_bytes, B, H, N, D, strides,
+                                                sm_scale, num_splits, stream);
+}
 
 int vqa_decode_default_splits(int B, int H, int N) { return vqa::decode::default_splits(B, H, N); }
 

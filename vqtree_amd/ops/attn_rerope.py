@@ -6,7 +6,7 @@ import math
 
 import torch
 
-from .attn_vq import apply_rope, rope_tables, rotate_half
+from .attn_vq import apply_rope, attn_exact_decode, rope_tables, rotate_half
 from .triton_fused_attn_rerope import attention
 from .triton_fused_local_attn import flash_attn_func as causal_window_attention
 
@@ -78,8 +78,8 @@ def rerope_attn_forward(query_states, key_states, value_states, position_ids, ca
     * short prefill: plain causal attention on the rotated operands (window kernel with the window covering
       everything);
     * generation (q_len == 1): the new key is appended (far keys re-rotated by the cache) and the query attends over
-      all cached keys; this single-row step is a torch scaled-dot-product call, the role a third-party flash
-      attention call plays in the reference (ops/attn_rerope.py:279-286).
+      all cached keys with the exact-key streaming decode kernel (a third-party flash attention call in the
+      reference, ops/attn_rerope.py:279-286).
     """
     assert isinstance(cache, ReRoPECache), "ReRoPECache is required"
     B, H, q_len, D = query_states.shape
@@ -107,5 +107,5 @@ def rerope_attn_forward(query_states, key_states, value_states, position_ids, ca
         out = causal_window_attention(q.transpose(1, 2), keys.transpose(1, 2), values.transpose(1, 2), q_len,
                                       softmax_scale=scale)
         return out.reshape(B, q_len, H * D).contiguous()
-    out = torch.nn.functional.scaled_dot_product_attention(q, keys, values, scale=scale)
+    out = attn_exact_decode(q, keys, values, softmax_scale=scale)
     return out.transpose(1, 2).reshape(B, q_len, H * D).contiguous()

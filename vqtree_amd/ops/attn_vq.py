@@ -68,6 +68,51 @@ def attn_vq_decode(q, k_codes, codebooks, v, *, softmax_scale=None, return_lse=F
     return (out, lse) if return_lse else out
 
 
+def attn_exact_decode(q, k, v, *, softmax_scale=None, return_lse=False, num_splits=0):
+    """seqlen_q == 1 attention over exact keys: q [B,H,1,D], k / v [B,H,N,D] -> out [B,H,1,D] (and lse [B,H,1] fp32,
+    base 2).  No mask: the single query sees every key."""
+    lib = _lib.load()
+    _lib.require_gpu(q, k, v)
+    q, k, v = (_last_dim_contiguous(x) for x in (q, k, v))
+    B, H, one, D = q.shape
+    N = k.shape[2]
+    assert one == 1 and k.shape == (B, H, N, D) and v.shape == (B, H, N, D)
+    assert q.dtype == k.dtype == v.dtype and q.dtype in _SUFFIX, "Only support fp16 and bf16"
+    softmax_scale = softmax_scale or 1.0 / math.sqrt(D)
+    out = torch.empty((B, H, 1, D), dtype=q.dtype, device=q.device)
+    lse = torch.empty((B, H, 1), dtype=torch.float32, device=q.device) if return_lse else None
+    S = num_splits if num_splits > 0 else lib.vqa_decode_default_splits(B, H, N)
+    ws = torch.empty(lib.vqa_decode_exact_workspace_bytes(B, H, N, D, S), dtype=torch.uint8, device=q.device)
+    strides = _lib.strides_array(q.stride(0), q.stride(1), k.stride(0), k.stride(1), k.stride(2), v.stride(0),
+                                 v.stride(1), v.stride(2), out.stride(0), out.stride(1))
+    with torch.cuda.device(q.device):
+        rc = getattr(lib, "vqa_decode_exact_" + _SUFFIX[q.dtype])(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), None if lse is None else lse.data_ptr(),
+            ws.data_ptr(), ws.numel(), B, H, N, D, strides, softmax_scale, S, _lib.current_stream(q.device))
+    _lib.check(rc)
+    return (out, lse) if return_lse else out
+
+
+def attn_vq_decode_windowed(q, k_codes, codebooks, v, k_window, *, softmax_scale=None):
+    """seqlen_q == 1 attention with an exact window: the last `k_window.shape[2]` keys are scored exactly
+    (k_window [B,H,W,D]), every earlier key through its codes; v [B,H,N,D] covers both.  Two streaming passes over
+    disjoint key ranges and one base-2 log-sum-exp merge."""
+    from .triton_fused_vq_attn import merge_state_in_place
+
+    B, H, _, D = q.shape
+    N, W = v.shape[2], k_window.shape[2]
+    assert 0 < W <= N and k_codes.shape[2] >= N - W
+    if W == N:
+        return attn_exact_decode(q, k_window, v, softmax_scale=softmax_scale)
+    far = N - W
+    o_far, l_far = attn_vq_decode(q, k_codes[:, :, :far], codebooks, v[:, :, :far], softmax_scale=softmax_scale,
+                                  return_lse=True)
+    o_win, l_win = attn_exact_decode(q, k_window, v[:, :, far:], softmax_scale=softmax_scale, return_lse=True)
+    # merge layout [rows, heads, D] / [rows, heads] with one row
+    merge_state_in_place(o_far.view(1, B * H, D), l_far.view(1, B * H), o_win.view(1, B * H, D), l_win.view(1, B * H))
+    return o_far
+
+
 def attn_vq_prefill(q, k_codes, codebooks, v, *, k_exact=None, window_size=0, causal=True, softmax_scale=None,
                     return_lse=False, boundary_mode="block", q2=None, k2=None):
     """Prefill attention (seqlen_q == seqlen_k) over additive-quantiser key codes, optionally with an exact window.
