@@ -110,3 +110,16 @@ def test_encoder_preprocessing_rope_reject_bad_arguments_before_any_launch(lib):
     merge = lambda lse=16, out=16: lib.vqa_vqcount_merge_bf16(16, 16, 16, 16, 16, out, lse, 1, 1, 256, 128, 128, s17,
                                                               64, 1.0, None)
     assert merge(lse=None) == -1 and merge(out=None) == -1          # the state to merge into is required
+
+
+def test_exact_decode_rejects_bad_arguments_before_any_launch(lib):
+    s10 = _lib.strides_array(*([8] * 10))
+    need = lib.vqa_decode_exact_workspace_bytes(2, 4, 5000, 128, 4)
+    assert need >= 8 * 4 * 130 * 4 and need % 256 == 0 and lib.vqa_decode_exact_workspace_bytes(2, 4, 0, 128, 4) == 0
+    call = lambda q=16, k=16, v=16, out=16, ws=256, ws_bytes=1 << 20, N=5000, D=128: lib.vqa_decode_exact_bf16(
+        q, k, v, out, None, ws, ws_bytes, 2, 4, N, D, s10, 1.0, 4, None)
+    assert call(k=None) == -1 and call(ws=None) == -1
+    assert call(N=0) == -2
+    assert call(D=96) == -3
+    assert call(v=24) == -5 and call(ws=64) == -5
+    assert call(ws_bytes=need - 1) == -6
