@@ -122,6 +122,45 @@ def test_decode_harness_matches_dense_reference():
         r = r - cb[1, m, int(codes[0, 1, 2, m])].float()
 
 
+def test_decode_harness_with_exact_window_matches_dense_reference():
+    """Same loop with the last W keys kept exactly: coded far keys scored with the clamped query, window keys with
+    the query at its true position, against dense fp32 softmax over [reconstructed far keys ; window keys].  W = 4
+    and 12 steps make the 2W-row window buffer compact itself during the test."""
+    from vqtree_amd.decode_harness import VQDecodeModel
+
+    def dense_attention(q_far, q_win, codes, codebooks, v, k_win, softmax_scale):
+        n, w = v.shape[2], k_win.shape[2]
+        k_hat = oracle.reconstruct_keys(codes[:, :, : n - w].cpu(), codebooks.cpu())
+        s_far = q_far.float().cpu() @ k_hat.transpose(-1, -2)
+        s_win = q_win.float().cpu() @ k_win.float().cpu().transpose(-1, -2)
+        scores = torch.cat([s_far, s_win], dim=-1) * softmax_scale
+        out, _ = oracle.attend(scores, torch.ones(1, n, dtype=torch.bool), v.float().cpu())
+        return out.to(q_far.dtype).cuda()
+
+    kw = dict(layers=2, hidden=256, heads=2, head_dim=128, ffn=512, vocab=1000, n_codebooks=4, window=128,
+              capacity=400, batch=2, exact_window=4)
+    a, b = VQDecodeModel(**kw), VQDecodeModel(**kw)
+    a.fill_random_context(300), b.fill_random_context(300)
+    tok = torch.tensor([5, 42], device="cuda")
+    for step in range(12):
+        ta, la = a.step(tok, return_logits=True)
+        tb, lb = b.step(tok, attention=dense_attention, return_logits=True)
+        assert (la.float() - lb.float()).abs().max() <= 2e-2 * max(1.0, float(lb.float().abs().max())), step
+        # layer 0 sees identical inputs in both models: its window rows must agree bit for bit
+        assert torch.equal(a.layers[0]["kwin"][:, :, a.kwin_len - 4: a.kwin_len],
+                           b.layers[0]["kwin"][:, :, b.kwin_len - 4: b.kwin_len])
+        tok = tb
+    assert a.length == 312 and a.kwin_len <= 8
+    # a cache shorter than the window is plain exact attention
+    c = VQDecodeModel(**dict(kw, exact_window=64))
+    c.fill_random_context(10)
+    d = VQDecodeModel(**dict(kw, exact_window=64))
+    d.fill_random_context(10)
+    _, lc = c.step(tok, return_logits=True)
+    _, ld = d.step(tok, attention=dense_attention, return_logits=True)
+    assert (lc.float() - ld.float()).abs().max() <= 2e-2 * max(1.0, float(ld.float().abs().max()))
+
+
 def test_rerope_caller_routes():
     """Attention core of the ReRoPE module: long prefill through the full ReRoPE kernel against the dense oracle,
     cache contents after it, a short prefill (plain causal) and a generation step against dense softmax over the

@@ -4,8 +4,10 @@ unimplemented).
 
 Every layer keeps, per (batch, head): the additive-quantiser codes of its keys `[B,H,cap,M] uint8` and the values
 `[B,H,cap,D]`.  A step projects the new token, rotates q to the clamped ReRoPE position, encodes the new key greedily
-against the layer's codebooks (residual, nearest codeword; HIP encoder), appends code and value, and attends over the whole cache
-with the HIP decode kernel.  The linear layers are plain torch matmuls (weights ~ N(0, 0.02)): they are plumbing around
+against the layer's codebooks (residual, nearest codeword; HIP encoder), appends code and value, and attends over the
+whole cache with the HIP decode kernel.  With `exact_window = W` the last W keys are kept exactly as well (rotated at
+their true positions) and scored with the query at its true position; the coded and the exact part are merged by
+log-sum-exp.  The linear layers are plain torch matmuls (weights ~ N(0, 0.02)): they are plumbing around
 the attention path, which is what this harness measures.
 
     python -m vqtree_amd.decode_harness --layers 32 --context 65536 --batch 4 --steps 128
@@ -17,7 +19,7 @@ import time
 
 import torch
 
-from .ops.attn_vq import attn_vq_decode, rope_tables, rotate_half
+from .ops.attn_vq import attn_exact_decode, attn_vq_decode, attn_vq_decode_windowed, rope_tables, rotate_half
 from .ops.mini_vq import RESIDUAL, encode_keys
 
 
@@ -31,11 +33,12 @@ class VQDecodeModel:
     """Random-init Llama-2-shaped decoder (RMSNorm, rotary attention over a VQ key cache, SwiGLU MLP)."""
 
     def __init__(self, layers, hidden, heads, head_dim, ffn, vocab, n_codebooks, window, capacity, batch,
-                 dtype=torch.bfloat16, device="cuda", seed=5, cb_std=0.35):
+                 dtype=torch.bfloat16, device="cuda", seed=5, cb_std=0.35, exact_window=0):
         g = torch.Generator(device=device).manual_seed(seed)
         w = lambda *s: (torch.randn(*s, generator=g, device=device, dtype=torch.float32) * 0.02).to(dtype)
         self.L, self.hidden, self.H, self.D, self.M = layers, hidden, heads, head_dim, n_codebooks
         self.window, self.capacity, self.B = window, capacity, batch
+        self.exact_window = exact_window  # 0: every key is scored through its codes; W > 0: the last W keys exactly
         self.dtype, self.device = dtype, device
         self.embed = w(vocab, hidden)
         self.lm_head = w(hidden, vocab)
@@ -47,10 +50,16 @@ class VQDecodeModel:
                 codebooks=(torch.randn(heads, n_codebooks, 256, head_dim, generator=g, device=device) * cb_std).to(dtype),
                 codes=torch.empty(batch, heads, capacity, n_codebooks, dtype=torch.uint8, device=device),
                 values=torch.empty(batch, heads, capacity, head_dim, dtype=dtype, device=device),
+                # the most recent exact keys (rotated at their true positions): rows [kwin_len - w, kwin_len) of a
+                # 2W-row buffer that is compacted when it fills up, so the window is always one contiguous slice
+                kwin=(torch.empty(batch, heads, 2 * exact_window, head_dim, dtype=dtype, device=device)
+                      if exact_window else None),
             ))
         self.length = 0
-        cos, sin = rope_tables(head_dim, window + 2, dtype=dtype, device=device)
-        self.cos_w, self.sin_w = cos[window + 1], sin[window + 1]  # every far key is seen at the clamped position
+        self.kwin_len = 0
+        self.cos, self.sin = rope_tables(head_dim, max(capacity, window + 2), dtype=dtype, device=device)
+        # every far key is seen at the clamped position
+        self.cos_w, self.sin_w = self.cos[window + 1], self.sin[window + 1]
 
     def fill_random_context(self, n_tokens, seed=6):
         """Synthetic cache contents standing in for a prefill of n_tokens (random codes, V ~ N(0,1))."""
@@ -61,31 +70,57 @@ class VQDecodeModel:
             for b in range(self.B):
                 layer["values"][b, :, :n_tokens] = torch.randn(self.H, n_tokens, self.D, generator=g,
                                                                device=self.device).to(self.dtype)
+            if self.exact_window:
+                w = min(self.exact_window, n_tokens)
+                layer["kwin"][:, :, :w] = torch.randn(self.B, self.H, w, self.D, generator=g,
+                                                      device=self.device).to(self.dtype)
         self.length = n_tokens
+        self.kwin_len = min(self.exact_window, n_tokens)
 
     @staticmethod
     def _rms(x):
         return (x.float() * torch.rsqrt(x.float().pow(2).mean(-1, keepdim=True) + 1e-5)).to(x.dtype)
 
+    def _attend(self, layer, q_raw, n, attention, win_end):
+        """Attention of the new token (cache rows [0, n] are filled).  Coded keys are scored with the query at the
+        clamped position window + 1, exact window keys with the query at its true position n."""
+        scale = 1.0 / math.sqrt(self.D)
+        q_far = (q_raw * self.cos_w + rotate_half(q_raw) * self.sin_w).unsqueeze(2)  # [B,H,1,D]
+        codes, values = layer["codes"][:, :, : n + 1], layer["values"][:, :, : n + 1]
+        if not self.exact_window:
+            return (attention or attn_vq_decode)(q_far, codes, layer["codebooks"], values, softmax_scale=scale)
+        w = min(self.exact_window, n + 1)
+        k_win = layer["kwin"][:, :, win_end - w: win_end]
+        q_win = (q_raw * self.cos[n] + rotate_half(q_raw) * self.sin[n]).unsqueeze(2)
+        if attention is not None:
+            return attention(q_far, q_win, codes, layer["codebooks"], values, k_win, softmax_scale=scale)
+        if w == n + 1:
+            return attn_exact_decode(q_win, k_win, values, softmax_scale=scale)
+        return attn_vq_decode_windowed(q_far, codes, layer["codebooks"], values, k_win, softmax_scale=scale,
+                                       q_window=q_win)
+
     def step(self, tokens, attention=None, return_logits=False, events=None):
         """One greedy decode step for token ids [B]; returns next token ids [B] (and the logits).  `attention`
         overrides the attention operator (tests pass a dense reference)."""
-        attention = attention or attn_vq_decode
         B, H, D = self.B, self.H, self.D
         n = self.length
+        if self.exact_window and self.kwin_len == 2 * self.exact_window:  # compact the window buffer
+            for layer in self.layers:
+                layer["kwin"][:, :, : self.exact_window] = layer["kwin"][:, :, self.exact_window:].clone()
+            self.kwin_len = self.exact_window
         x = self.embed[tokens]  # [B, hidden]
         for layer in self.layers:
             h = self._rms(x)
             qkv = (h @ layer["wqkv"]).view(B, 3, H, D)
             q, k, v = qkv[:, 0], qkv[:, 1], qkv[:, 2]  # [B,H,D]
-            q2 = (q * self.cos_w + rotate_half(q) * self.sin_w).unsqueeze(2)  # [B,H,1,D]
             layer["codes"][:, :, n] = encode_residual(k.unsqueeze(2), layer["codebooks"])[:, :, 0]
             layer["values"][:, :, n] = v
+            if self.exact_window:
+                layer["kwin"][:, :, self.kwin_len] = k * self.cos[n] + rotate_half(k) * self.sin[n]
             if events is not None:
                 events.append(torch.cuda.Event(enable_timing=True))
                 events[-1].record()
-            o = attention(q2, layer["codes"][:, :, : n + 1], layer["codebooks"], layer["values"][:, :, : n + 1],
-                          softmax_scale=1.0 / math.sqrt(D))
+            o = self._attend(layer, q, n, attention, self.kwin_len + 1)
             if events is not None:
                 events.append(torch.cuda.Event(enable_timing=True))
                 events[-1].record()
@@ -94,22 +129,25 @@ class VQDecodeModel:
             gate, up = (h @ layer["w_gate_up"]).chunk(2, dim=-1)
             x = x + (torch.nn.functional.silu(gate) * up) @ layer["w_down"]
         self.length = n + 1
+        self.kwin_len += 1 if self.exact_window else 0
         logits = self._rms(x) @ self.lm_head
         return (logits.argmax(-1), logits) if return_logits else logits.argmax(-1)
 
     def attention_bytes_per_step(self):
-        """Algorithmic bytes of the attention path per token step: per layer codes + V + codebooks + q/out."""
+        """Algorithmic bytes of the attention path per token step: per layer codes of the coded keys + V + exact
+        window keys + codebooks + q/out."""
         e = 2
         n = self.length
-        per_layer = self.B * self.H * n * self.M + e * self.B * self.H * n * self.D + e * self.H * self.M * 256 * self.D \
-            + 2 * e * self.B * self.H * self.D
+        w = min(self.exact_window, n)
+        per_layer = self.B * self.H * (n - w) * self.M + e * self.B * self.H * n * self.D \
+            + e * self.B * self.H * w * self.D + e * self.H * self.M * 256 * self.D + 2 * e * self.B * self.H * self.D
         return self.L * per_layer
 
 
 def run(layers=32, hidden=4096, heads=32, head_dim=128, ffn=11008, vocab=32000, n_codebooks=4, context=65536, batch=4,
-        steps=128, warmup=4, window=1024, device="cuda"):
+        steps=128, warmup=4, window=1024, exact_window=0, device="cuda"):
     model = VQDecodeModel(layers, hidden, heads, head_dim, ffn, vocab, n_codebooks, window, context + steps + warmup,
-                          batch, device=device)
+                          batch, device=device, exact_window=exact_window)
     model.fill_random_context(context)
     g = torch.Generator(device=device).manual_seed(7)
     tokens = torch.randint(0, vocab, (batch,), generator=g, device=device)
@@ -130,19 +168,21 @@ def run(layers=32, hidden=4096, heads=32, head_dim=128, ffn=11008, vocab=32000, 
     attn_us = sum(events[i].elapsed_time(events[i + 1]) for i in range(0, len(events), 2)) / steps * 1e3
     return {
         "workload": f"{layers}-layer Llama-2-7B-shaped greedy decode, batch {batch}, context {context}, VQ key cache "
-                    f"{n_codebooks}x256 per layer, {steps} steps",
+                    f"{n_codebooks}x256 per layer, " + (f"last {exact_window} keys exact, " if exact_window else "")
+                    + f"{steps} steps",
         "us_per_step": round(us, 1),
         "attention_us_per_step": round(attn_us, 1),
         "attention_bytes_per_step": bytes_mid,
         "attention_GBps": round(bytes_mid / (attn_us * 1e-6) / 1e9, 1),
         "attention_hbm_frac": round(bytes_mid / (attn_us * 1e-6) / 8e12, 4),
         "note": "us_per_step is whole-step wall time (projections, MLP, key encoder, attention); attention_us_per_step "
-                "sums HIP-event intervals around the attention calls of all layers (3 kernels each)",
+                "sums HIP-event intervals around the attention calls of all layers (3 kernels each; 6 with an exact window)",
     }
 
 
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
-    for name, default in (("layers", 32), ("context", 65536), ("batch", 4), ("steps", 128), ("warmup", 4)):
+    for name, default in (("layers", 32), ("context", 65536), ("batch", 4), ("steps", 128), ("warmup", 4),
+                          ("exact_window", 0)):
         ap.add_argument("--" + name, type=int, default=default)
     print(json.dumps(run(**vars(ap.parse_args()))))

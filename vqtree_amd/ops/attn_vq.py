@@ -93,21 +93,23 @@ def attn_exact_decode(q, k, v, *, softmax_scale=None, return_lse=False, num_spli
     return (out, lse) if return_lse else out
 
 
-def attn_vq_decode_windowed(q, k_codes, codebooks, v, k_window, *, softmax_scale=None):
+def attn_vq_decode_windowed(q, k_codes, codebooks, v, k_window, *, softmax_scale=None, q_window=None):
     """seqlen_q == 1 attention with an exact window: the last `k_window.shape[2]` keys are scored exactly
-    (k_window [B,H,W,D]), every earlier key through its codes; v [B,H,N,D] covers both.  Two streaming passes over
-    disjoint key ranges and one base-2 log-sum-exp merge."""
+    (k_window [B,H,W,D], with `q_window` when the window uses another query, e.g. another rotary position), every
+    earlier key through its codes; v [B,H,N,D] covers both.  Two streaming passes over disjoint key ranges and one
+    base-2 log-sum-exp merge."""
     from .triton_fused_vq_attn import merge_state_in_place
 
     B, H, _, D = q.shape
     N, W = v.shape[2], k_window.shape[2]
     assert 0 < W <= N and k_codes.shape[2] >= N - W
+    q_window = q if q_window is None else q_window
     if W == N:
-        return attn_exact_decode(q, k_window, v, softmax_scale=softmax_scale)
+        return attn_exact_decode(q_window, k_window, v, softmax_scale=softmax_scale)
     far = N - W
     o_far, l_far = attn_vq_decode(q, k_codes[:, :, :far], codebooks, v[:, :, :far], softmax_scale=softmax_scale,
                                   return_lse=True)
-    o_win, l_win = attn_exact_decode(q, k_window, v[:, :, far:], softmax_scale=softmax_scale, return_lse=True)
+    o_win, l_win = attn_exact_decode(q_window, k_window, v[:, :, far:], softmax_scale=softmax_scale, return_lse=True)
     # merge layout [rows, heads, D] / [rows, heads] with one row
     merge_state_in_place(o_far.view(1, B * H, D), l_far.view(1, B * H), o_win.view(1, B * H, D), l_win.view(1, B * H))
     return o_far
