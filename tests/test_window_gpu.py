@@ -164,6 +164,27 @@ def test_vq_prefill_with_exact_window(B, H, N, D, M, W, with_rerope, boundary_mo
     assert_close_lse(lse, want_lse, atol=1e-2)
 
 
+@pytest.mark.parametrize("with_rerope", [False, True])
+def test_vq_prefill_fp16(with_rerope):
+    """The fp16 instantiation of the fused prefill (two-pair and three-pair kernels), strided [B,N,H,D]-backed q/k/v."""
+    _say(f"vq prefill fp16 rerope={with_rerope}")
+    B, H, N, D, M, W = 2, 2, 700, 128, 4, 256
+    mk = lambda seed: _bnhd(_randn(B, H, N, D, seed=seed, std=0.7, dtype=torch.float16)).transpose(1, 2)
+    q, k, v, q2, k2 = (mk(70 + s) for s in range(5))
+    cb = _randn(H, M, 256, D, seed=75, std=0.3, dtype=torch.float16)
+    codes = _codes(B, H, N, M, seed=76)
+    kw = dict(k_exact=k, window_size=W)
+    if with_rerope:
+        kw.update(q2=q2, k2=k2)
+    want, want_lse = oracle.attn_vq_prefill(q, codes, cb, v, **kw)
+    kw = {n: (t.cuda() if torch.is_tensor(t) else t) for n, t in kw.items()}
+    out, lse = attn_vq_prefill(q.cuda(), codes.cuda(), cb.cuda(), v.cuda(), return_lse=True, **kw)
+    torch.cuda.synchronize()
+    assert out.dtype == torch.float16
+    assert_close_16(out, want, "vq prefill fp16")
+    assert_close_lse(lse, want_lse, atol=1e-2)
+
+
 def test_vq_prefill_far_boundary_is_exact():
     """Mask/source check with little rounding slack: far keys score 1 (weight e), exact keys score 0 (weight 1), V rows
     are position markers; a key taken from the wrong side moves its output element by ~1e-3, rounding by ~1e-5."""
