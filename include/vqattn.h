@@ -7,7 +7,9 @@
  *   - allocates nothing and keeps no mutable global state (scratch comes in through `workspace`),
  *   - returns VQA_OK (0) or a negative vqa_status; it never throws or aborts.
  * Tensors are addressed as base + sum(index_i * stride_i) in ELEMENTS of their own type; the innermost
- * (head_dim / codebook index M) stride must be 1.  Head dims: 64 and 128.
+ * (head_dim / codebook index M) stride must be 1.  Head dims of the attention entry points: 64 and 128 (the encoder,
+ * preprocessing and rotary entry points state their own limits).  The count kernel needs 64.5 KB of LDS at head dim
+ * 128 and raises its dynamic-LDS limit with hipFuncSetAttribute on every call; nothing else touches process state.
  *
  * Log-sum-exp values are base 2 of the scaled scores, lse2 = log2(sum_j exp(s_ij * sm_scale)), the convention of
  * the reference kernels (ops/triton_fused_vq_attn.py:179, ops/triton_fused_local_attn_rerope.py:214-216).
