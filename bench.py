@@ -23,7 +23,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
 DECODE_MAIN_KERNEL_TRAFFIC_BYTES = 4_380_977_000
 
 
-def cpu_baseline(case, units=32, repeats=3):
+def cpu_baseline(case, units=256, repeats=5):
     """The fp32 PyTorch oracle timed on the host cores over `units` (batch, head) problems of the same workload.
 
     Returns the equivalent HBM rate (algorithmic bytes of the sampled units / time) so it is comparable with `value`.
