@@ -248,15 +248,24 @@ __global__ __launch_bounds__(kThreads, 2) void window_kernel(Params p) {
         wait_tile_loads();
         __syncthreads();
         f32x16_t s[2];
+        auto extra_pair = [&](int src) {  // pair `src` is scored in this tile besides the main one
+            if (MODE == kVqPrefill2 && src == 1) return false;
+            if (MODE != kVqPrefill && MODE != kVqPrefill2 && src == 2) return false;
+            return src != tg.main && ((tg.need >> src) & 1) != 0;
+        };
+        // the first extra pair's K tile is requested before the main product so that the product hides its latency
+        int early = -1;
+        if constexpr (kDual) {
+            early = extra_pair(0) ? 0 : (extra_pair(1) ? 1 : (extra_pair(2) ? 2 : -1));
+            if (early >= 0) k_copy.load(nxt_k, k_ptr(early), k_stride(early), n0, p.N);
+        }
         hold_q(kDual && tg.main != 0 ? 1 : 0);
         qk_mma<Tag, D>(s, q, cur_k, lane);
         if constexpr (kDual) {
             // the other pairs, one K tile at a time through the (still free) K buffer of the next tile
             for (int src = 0; src < 3; ++src) {
-                if (MODE == kVqPrefill2 && src == 1) continue;
-                if (MODE != kVqPrefill && MODE != kVqPrefill2 && src == 2) continue;
-                if (src == tg.main || !((tg.need >> src) & 1)) continue;
-                k_copy.load(nxt_k, k_ptr(src), k_stride(src), n0, p.N);
+                if (!extra_pair(src)) continue;
+                if (src != early) k_copy.load(nxt_k, k_ptr(src), k_stride(src), n0, p.N);
                 hold_q(src == 0 ? 0 : 1);
                 wait_tile_loads();
                 __syncthreads();
