@@ -241,7 +241,7 @@ int vqa_decode_exact_f16(const void* q, const void* k, const void* v, void* out,
  *           codebooks offline (build_quantizer/120_build_additive_quantizer.py:23-32) and has no runtime encoder.
  *
  *   x [B,H,N,D]; codebooks [H,M,K,D], K % 32 == 0; codes [B,H,N,M] uint8 (nullable, needs K <= 256);
- *   ids [B,H,N,M] int64 (nullable); at least one output.  D in {16,32,64,128}.
+ *   ids [B,H,N,M] int64 (nullable); at least one output.  D in {64,128}.
  *   strides[0..11] = x(b,h,n) codebooks(h,m,k) codes(b,h,n) ids(b,h,n); m is innermost in codes and ids.
  * ------------------------------------------------------------------------------------------------------------------ */
 #define VQA_ENCODE_NUM_STRIDES 12

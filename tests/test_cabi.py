@@ -83,7 +83,7 @@ def test_encoder_preprocessing_rope_reject_bad_arguments_before_any_launch(lib):
         x, cb, codes, ids, 1, 1, N, D, M, K, s12, mode, 0, None)
     assert enc(x=None) == -1 and enc(codes=None, ids=None) == -1   # VQA_ERR_NULL_POINTER
     assert enc(N=0) == -2 and enc(K=250) == -2                      # VQA_ERR_BAD_SHAPE (K must be a multiple of 32)
-    assert enc(D=96) == -3                                          # VQA_ERR_UNSUPPORTED_HEAD_DIM
+    assert enc(D=96) == -3 and enc(D=32) == -3                      # VQA_ERR_UNSUPPORTED_HEAD_DIM
     assert enc(K=512) == -7 and enc(mode=2) == -7                   # uint8 codes need K <= 256; unknown mode
     assert enc(x=18) == -5                                          # VQA_ERR_MISALIGNED
 

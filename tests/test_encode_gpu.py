@@ -18,8 +18,8 @@ def _draw(shape, dtype, seed, std=1.0):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("B,H,N,D,K", [(2, 3, 300, 128, 256), (1, 2, 130, 64, 512), (2, 2, 1, 128, 128), (1, 1, 129, 16, 32),
-                                       (1, 2, 257, 32, 8192)])
+@pytest.mark.parametrize("B,H,N,D,K", [(2, 3, 300, 128, 256), (1, 2, 130, 64, 512), (2, 2, 1, 128, 128), (1, 1, 129, 64, 32),
+                                       (1, 2, 257, 64, 8192), (1, 1, 200, 128, 96)])
 def test_inner_product_search(dtype, B, H, N, D, K):
     print(f"encode: inner product {dtype} B{B} H{H} N{N} D{D} K{K}", flush=True)
     x, cb = _draw((B, H, N, D), dtype, 1), _draw((H, 1, K, D), dtype, 2)
@@ -64,7 +64,7 @@ def test_ties_take_the_first_codeword():
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("B,H,N,D,M,K", [(2, 2, 300, 128, 4, 256), (1, 3, 129, 64, 2, 256), (4, 2, 1, 128, 4, 256),
-                                         (1, 2, 70, 32, 8, 64)])
+                                         (1, 2, 70, 64, 8, 64), (1, 1, 333, 128, 3, 160)])
 def test_residual_encoder(dtype, B, H, N, D, M, K):
     print(f"encode: residual {dtype} B{B} H{H} N{N} D{D} M{M} K{K}", flush=True)
     x, cb = _draw((B, H, N, D), dtype, 7), _draw((H, M, K, D), dtype, 8, std=0.6)

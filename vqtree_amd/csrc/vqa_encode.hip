@@ -3,18 +3,20 @@
 //   mode 0 (inner product):   id_m = argmax_c <x, cb[h,m,c]>                       for every codebook m independently
 //   mode 1 (greedy residual): r = x;  id_m = argmax_c (<r, cb[h,m,c]> - |cb[h,m,c]|^2 / 2);  r -= cb[h,m,id_m]
 //
-// One workgroup = 4 waves x 32 keys of one (batch, head).  Scores are computed transposed, S^T = CB . R^T, with the
-// codebook chunk (128 codewords, staged in LDS) as the A operand and the keys as the B operand, so a lane owns one key
-// and sees 16 codeword scores per 32x32 block: the running argmax lives in registers.  The residual is kept in fp32 and
-// fed to the 16-bit MFMA as a (high, low) pair of 16-bit values, which reproduces fp32 inner products to ~2^-16.
-#include "vqa_common.h"
+// One workgroup = 4 waves x 32 keys of one (batch, head).  The codebooks stream through LDS in 64-codeword tiles with
+// the attention kernels' machinery (direct-to-LDS copies, XOR-swizzled rows, double buffering across tiles and
+// stages), and the scores are the same transposed product S^T = CB_tile . R^T: a lane owns one key and sees 2 x 16
+// codeword scores per tile, in increasing codeword order, so the running arg-max is two registers and the first
+// maximum wins ties.  The residual is kept in fp32 and fed to the 16-bit MFMA as a (high, low) pair of 16-bit
+// values, which reproduces fp32 inner products to ~2^-16.
+#include "vqa_flash.h"
 
 namespace vqa {
 namespace encode {
 
+using flash::kBN;
 constexpr int kThreads = 256;
 constexpr int kKeysPerBlock = 128;
-constexpr int kChunk = 128;  // codewords staged per pass
 
 struct Params {
     const uint16_t* x;
@@ -30,24 +32,34 @@ struct Params {
 };
 
 template <typename Tag, int D>
-__global__ __launch_bounds__(kThreads) void encode_kernel(Params p) {
+__global__ __launch_bounds__(kThreads, 2) void encode_kernel(Params p) {
+    typedef flash::Geom<D> G;
     typedef typename Elem<Tag>::vec8 vec8;
-    constexpr int kSteps = D / 16;      // MFMA k-steps
-    constexpr int kRowElems = D + 8;    // padded LDS row: 16-byte reads of 16 consecutive rows hit distinct banks
-    constexpr int kChunksPerRow = D / 8;
-    __shared__ __attribute__((aligned(16))) uint16_t s_cb[kChunk * kRowElems];
-    __shared__ float s_norm[kChunk];
+    constexpr int kSteps = D / 16;
+    __shared__ __attribute__((aligned(1024))) char s_cb[2][G::kTileBytes];
+    __shared__ __attribute__((aligned(16))) float s_norm[kBN];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int half = lane >> 5;
     const int bh = blockIdx.y;
     const int b = bh / p.H, h = bh % p.H;
     const int key = blockIdx.x * kKeysPerBlock + wave * 32 + (lane & 31);
     const int key_c = min(key, p.N - 1);
+    const uint16_t* cb_h = p.cb + h * p.cb_sh;
 
-    // this lane's slice of its key: elements ks*16 + half*8 + [0, 8)
+    flash::TileCopy<D, false> copy;
+    copy.init(wave, lane);
+    const int tiles_per_stage = (p.K + kBN - 1) / kBN;
+    const int n_tiles = p.M * tiles_per_stage;
+    auto request = [&](int idx, int buf) {  // tile idx = (codebook m, 64-codeword tile t); rows past K repeat row K-1
+        const int m = idx / tiles_per_stage, t = idx % tiles_per_stage;
+        copy.load(s_cb[buf], cb_h + m * p.cb_sm, p.cb_sk, t * kBN, p.K);
+    };
+    request(0, 0);
+
+    // this lane's slice of its key: elements ks*16 + half*8 + [0, 8), the B-operand layout of the score product
     float r[kSteps * 8];
     {
         const uint16_t* xp = p.x + b * p.x_sb + h * p.x_sh + (int64_t)key_c * p.x_sn + half * 8;
@@ -63,12 +75,13 @@ __global__ __launch_bounds__(kThreads) void encode_kernel(Params p) {
         }
     }
 
+    int idx = 0;
     for (int m = 0; m < p.M; ++m) {
-        const uint16_t* cbm = p.cb + h * p.cb_sh + m * p.cb_sm;
+        const uint16_t* cbm = cb_h + m * p.cb_sm;
         const bool with_low = p.mode == 1 && m > 0;  // the residual is no longer a 16-bit value after one subtraction
 
         // split the fp32 residual into the two 16-bit MFMA operands
-        vec8 hi[kSteps], lo[kSteps];
+        flash::QFrag<Tag, D> hi, lo;
 #pragma unroll
         for (int ks = 0; ks < kSteps; ++ks) {
             uint32_t wh[4], wl[4];
@@ -79,55 +92,70 @@ __global__ __launch_bounds__(kThreads) void encode_kernel(Params p) {
                 wh[e] = Elem<Tag>::pack2(h0, h1);
                 wl[e] = Elem<Tag>::pack2(a0 - h0, a1 - h1);
             }
-            const uint4 vh = make_uint4(wh[0], wh[1], wh[2], wh[3]);
-            const uint4 vl = make_uint4(wl[0], wl[1], wl[2], wl[3]);
-            hi[ks] = __builtin_bit_cast(vec8, vh);
-            lo[ks] = __builtin_bit_cast(vec8, vl);
+            const flash::u32x4_t vh = {wh[0], wh[1], wh[2], wh[3]};
+            const flash::u32x4_t vl = {wl[0], wl[1], wl[2], wl[3]};
+            hi.f[ks] = __builtin_bit_cast(vec8, vh);
+            lo.f[ks] = __builtin_bit_cast(vec8, vl);
         }
 
         float best = -INFINITY;
         int best_i = 0;
-        for (int c0 = 0; c0 < p.K; c0 += kChunk) {
-            const int rows = min(kChunk, p.K - c0);
-            __syncthreads();  // the previous chunk is no longer read
-            for (int i = tid; i < rows * kChunksPerRow; i += kThreads) {
-                const int row = i / kChunksPerRow, col = i % kChunksPerRow;
-                *reinterpret_cast<uint4*>(&s_cb[row * kRowElems + col * 8]) =
-                    *reinterpret_cast<const uint4*>(cbm + (int64_t)(c0 + row) * p.cb_sk + col * 8);
-            }
-            __syncthreads();
+        for (int t = 0; t < tiles_per_stage; ++t, ++idx) {
+            const int buf = idx & 1;
+            flash::wait_tile_loads();
+            __syncthreads();  // tile idx is complete in `buf`; every wave is done with the other buffer and s_norm
+            if (idx + 1 < n_tiles) request(idx + 1, buf ^ 1);
             if (p.mode == 1) {
-                if (tid < rows) {
-                    float acc = 0.f;
-                    for (int d = 0; d < D; ++d) {
-                        const float cv = Elem<Tag>::from_bits(s_cb[tid * kRowElems + d]);
-                        acc += cv * cv;
+                // |c|^2 / 2 of the tile's 64 codewords: 4 threads per row, 16-byte chunks through the row swizzle
+                constexpr int kCPT = G::kChunksPerRow / 4;  // chunks per thread
+                const int row = tid >> 2, part = tid & 3;
+                float acc = 0.f;
+#pragma unroll
+                for (int j = 0; j < kCPT; ++j) {
+                    const int chunk = (part * kCPT + j) ^ G::swz_k(row);
+                    const flash::u32x4_t w = *reinterpret_cast<const flash::u32x4_t*>(
+                        &s_cb[buf][row * G::kRowBytes + chunk * 16]);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const float lo16 = Elem<Tag>::from_bits((uint16_t)(w[e] & 0xffffu));
+                        const float hi16 = Elem<Tag>::from_bits((uint16_t)(w[e] >> 16));
+                        acc += lo16 * lo16 + hi16 * hi16;
                     }
-                    s_norm[tid] = 0.5f * acc;
                 }
+                acc += __shfl_xor(acc, 1, 64);
+                acc += __shfl_xor(acc, 2, 64);
+                if (part == 0) s_norm[row] = 0.5f * acc;
                 __syncthreads();
             }
-            for (int blk = 0; blk * 32 < rows; ++blk) {
-                f32x16_t acc = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-                const uint16_t* ap = &s_cb[(blk * 32 + (lane & 31)) * kRowElems + half * 8];
+            f32x16_t s[2];
+            flash::qk_mma<Tag, D>(s, hi, s_cb[buf], lane);
+            if (with_low) {
+                f32x16_t s2[2];
+                flash::qk_mma<Tag, D>(s2, lo, s_cb[buf], lane);
 #pragma unroll
-                for (int ks = 0; ks < kSteps; ++ks) {
-                    const vec8 a = *reinterpret_cast<const vec8*>(ap + ks * 16);
-                    acc = Elem<Tag>::mfma32(a, hi[ks], acc);
-                    if (with_low) acc = Elem<Tag>::mfma32(a, lo[ks], acc);
-                }
+                for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    const int cl = blk * 32 + 8 * (e / 4) + 4 * half + (e % 4);  // codeword within the chunk
-                    float s = acc[e];
-                    if (p.mode == 1) s -= s_norm[cl];
-                    if (p.round_scores) s = Elem<Tag>::round_keep_f32(s);
-                    if (s > best) {  // a lane visits its codewords in increasing order: the first maximum stays
-                        best = s;
-                        best_i = c0 + cl;
+                    for (int e = 0; e < 16; ++e) s[kb][e] += s2[kb][e];
+            }
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    // registers 4g .. 4g+3 of block kb are codewords kb*32 + 8g + 4*half + 0..3 of the tile
+                    const int cl0 = kb * 32 + 8 * g + 4 * half;
+                    f32x4_t nrm = {0.f, 0.f, 0.f, 0.f};
+                    if (p.mode == 1) nrm = *reinterpret_cast<const f32x4_t*>(&s_norm[cl0]);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        float sc = s[kb][4 * g + e] - nrm[e];
+                        if (p.round_scores) sc = Elem<Tag>::round_keep_f32(sc);
+                        const int c = t * kBN + cl0 + e;
+                        if (c < p.K && sc > best) {  // a lane meets its codewords in increasing order: first maximum
+                            best = sc;
+                            best_i = c;
+                        }
                     }
                 }
-            }
         }
         // the two half-waves hold disjoint codewords of the same key
         const float o_s = __shfl_xor(best, 32, 64);
@@ -180,8 +208,6 @@ int encode(const void* x, const void* codebooks, uint8_t* codes, int64_t* ids, i
         return VQA_ERR_MISALIGNED;
     const dim3 grid((N + kKeysPerBlock - 1) / kKeysPerBlock, B * H);
     switch (D) {
-        case 16: hipLaunchKernelGGL((encode_kernel<Tag, 16>), grid, dim3(kThreads), 0, stream, p); break;
-        case 32: hipLaunchKernelGGL((encode_kernel<Tag, 32>), grid, dim3(kThreads), 0, stream, p); break;
         case 64: hipLaunchKernelGGL((encode_kernel<Tag, 64>), grid, dim3(kThreads), 0, stream, p); break;
         case 128: hipLaunchKernelGGL((encode_kernel<Tag, 128>), grid, dim3(kThreads), 0, stream, p); break;
         default: return VQA_ERR_UNSUPPORTED_HEAD_DIM;
