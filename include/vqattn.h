@@ -283,17 +283,19 @@ int vqa_preprocess_f16(const int64_t* ids, const void* v, int64_t* cnt, void* cn
  * (apply_rotary_pos_emb and the clamped query at ops/attn_vq.py:402-407; ops/attn_rerope.py:160-180).
  *
  *   x, out [B,H,N,D]; position_ids [B,N] int64, or null to rotate every row to `fixed_pos`; cos, sin [n_pos, D] with
- *   row stride table_stride.  D % 16 == 0.  strides[0..7] = x(b,h,n) position_ids(b,n) out(b,h,n).
+ *   row stride table_stride.  out_fixed (nullable, only with position_ids; addressed with out's strides) receives the
+ *   same rows rotated to `fixed_pos` from the same pass over x -- the clamped ReRoPE query next to the true-position
+ *   one.  D % 16 == 0.  strides[0..7] = x(b,h,n) position_ids(b,n) out(b,h,n).
  * ------------------------------------------------------------------------------------------------------------------ */
 #define VQA_ROPE_NUM_STRIDES 8
 
-int vqa_rope_bf16(const void* x, const int64_t* position_ids, const void* cos, const void* sin, void* out, int B,
-                  int H, int N, int D, int n_pos, int64_t table_stride, const int64_t* strides, int fixed_pos,
-                  vqa_stream_t stream);
+int vqa_rope_bf16(const void* x, const int64_t* position_ids, const void* cos, const void* sin, void* out,
+                  void* out_fixed, int B, int H, int N, int D, int n_pos, int64_t table_stride, const int64_t* strides,
+                  int fixed_pos, vqa_stream_t stream);
 
-int vqa_rope_f16(const void* x, const int64_t* position_ids, const void* cos, const void* sin, void* out, int B, int H,
-                 int N, int D, int n_pos, int64_t table_stride, const int64_t* strides, int fixed_pos,
-                 vqa_stream_t stream);
+int vqa_rope_f16(const void* x, const int64_t* position_ids, const void* cos, const void* sin, void* out,
+                 void* out_fixed, int B, int H, int N, int D, int n_pos, int64_t table_stride, const int64_t* strides,
+                 int fixed_pos, vqa_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -99,12 +99,13 @@ def test_encoder_preprocessing_rope_reject_bad_arguments_before_any_launch(lib):
     assert pre(ws_bytes=need - 1) == -6                             # VQA_ERR_WORKSPACE_TOO_SMALL
     assert pre(ws=128) == -5
 
-    rope = lambda x=16, pos=16, cos=16, sin=16, out=16, D=128, n_pos=64, fixed=0: lib.vqa_rope_bf16(
-        x, pos, cos, sin, out, 1, 1, 8, D, n_pos, 128, s8, fixed, None)
+    rope = lambda x=16, pos=16, cos=16, sin=16, out=16, out2=None, D=128, n_pos=64, fixed=0: lib.vqa_rope_bf16(
+        x, pos, cos, sin, out, out2, 1, 1, 8, D, n_pos, 128, s8, fixed, None)
     assert rope(x=None) == -1 and rope(cos=None) == -1
     assert rope(D=24) == -3
     assert rope(pos=None, fixed=64) == -7 and rope(pos=None, fixed=-1) == -7   # fixed position outside the tables
     assert rope(out=20) == -5
+    assert rope(pos=None, out2=16) == -7 and rope(out2=16, fixed=99) == -7      # second output: per-row form only
 
     s17 = _lib.strides_array(*([8] * 17))
     merge = lambda lse=16, out=16: lib.vqa_vqcount_merge_bf16(16, 16, 16, 16, 16, out, lse, 1, 1, 256, 128, 128, s17,

@@ -133,3 +133,5 @@ def test_rotary_kernel_is_bit_exact(dtype, B, H, N, D):
     got_fixed = A.apply_rope(x.cuda(), cos.cuda(), sin.cuda(), 33).cpu()
     assert torch.equal(got_fixed, oracle.apply_rope(x, cos, sin, 33))
     assert torch.equal(A.apply_rope(x.cuda(), cos.cuda(), sin.cuda(), 0).cpu(), x)  # position 0 is the identity
+    both = A.apply_rope(x.cuda(), cos.cuda(), sin.cuda(), pos.cuda(), also_fixed=33)  # one pass, two outputs
+    assert torch.equal(both[0].cpu(), got) and torch.equal(both[1].cpu(), got_fixed)

@@ -242,11 +242,12 @@ def rope_tables(head_dim, n_pos, base=10000.0, dtype=torch.float32, device=None)
     return have[0][:n_pos], have[1][:n_pos]
 
 
-def apply_rope(x, cos, sin, positions):
+def apply_rope(x, cos, sin, positions, also_fixed=None):
     """x * cos[p] + rotate_half(x) * sin[p] for x [B,H,N,D]; `positions` is a LongTensor [B,N] or one int for every
     row.  16-bit tensors on the GPU run the HIP rotary kernel, whose rounding (each product and the sum rounded to the
     element type) is that of this very expression evaluated on 16-bit tensors; anything else evaluates the expression
-    with torch operators."""
+    with torch operators.  `also_fixed = p` (with per-row positions) returns a pair: the rows at their own positions
+    and the same rows at the single position p, from one pass over x."""
     from .. import _lib
     from ._common import SUFFIX, bhn_strides, ptr
 
@@ -260,23 +261,29 @@ def apply_rope(x, cos, sin, positions):
             cos = cos.contiguous()
         out = torch.empty((B, H, N, D), dtype=x.dtype, device=x.device)
         fixed = isinstance(positions, int)
+        assert also_fixed is None or not fixed
+        out2 = torch.empty_like(out) if also_fixed is not None else None
         if not fixed:
             positions = positions.to(torch.int64)
             assert positions.shape == (B, N)
         strides = _lib.strides_array(*bhn_strides(x), *((0, 0) if fixed else (positions.stride(0), positions.stride(1))),
                                      *bhn_strides(out))
         with torch.cuda.device(x.device):
+            fixed_pos = positions if fixed else (int(also_fixed) if also_fixed is not None else 0)
             rc = getattr(lib, "vqa_rope_" + SUFFIX[x.dtype])(ptr(x), None if fixed else ptr(positions), ptr(cos),
-                                                             ptr(sin), ptr(out), B, H, N, D, cos.shape[0],
-                                                             cos.stride(0), strides, positions if fixed else 0,
+                                                             ptr(sin), ptr(out), ptr(out2), B, H, N, D, cos.shape[0],
+                                                             cos.stride(0), strides, fixed_pos,
                                                              _lib.current_stream(x.device))
         _lib.check(rc)
-        return out
+        return out if also_fixed is None else (out, out2)
     if isinstance(positions, int):
         c, s = cos[positions], sin[positions]
     else:
         c, s = cos[positions].unsqueeze(1), sin[positions].unsqueeze(1)  # [B,1,N,D]
-    return x * c + rotate_half(x) * s
+    out = x * c + rotate_half(x) * s
+    if also_fixed is None:
+        return out
+    return out, x * cos[also_fixed] + rotate_half(x) * sin[also_fixed]
 
 
 def rerope_operands(query_states, key_states, position_ids, window_length, rope_base=10000.0):
@@ -285,9 +292,8 @@ def rerope_operands(query_states, key_states, position_ids, window_length, rope_
     B, H, N, D = query_states.shape
     n_pos = max(int(position_ids.max()) + 1, window_length + 2)
     cos, sin = rope_tables(D, n_pos, rope_base, query_states.dtype, query_states.device)
-    q1 = apply_rope(query_states, cos, sin, position_ids)
+    q1, q2 = apply_rope(query_states, cos, sin, position_ids, also_fixed=window_length + 1)
     k1 = apply_rope(key_states, cos, sin, position_ids)
-    q2 = apply_rope(query_states, cos, sin, window_length + 1)
     return q1, k1, q2
 
 
