@@ -85,3 +85,36 @@ def test_local_rerope_benchmark_size_sampled_rows_and_prefix():
     out_half = local_rerope(q1[:, :half], q2[:, :half], k1[:, :half], k[:, :half], v[:, :half], W, scale)
     torch.cuda.synchronize()
     assert (out_half.float() - out[:, :half].float()).abs().max().item() <= 2e-2
+
+
+def test_reference_shaped_route_benchmark_length_sampled_rows():
+    """The whole caller chain (encoder -> preprocessing kernels -> rotary -> window kernel -> count kernel with fused
+    merge) at 8192 tokens, window 1024, 512 codewords: sampled rows against the per-query statement of the reference's
+    slow path (ops/attn_vq.py:305-333): exact keys in the window, raw keys with the clamped query on the strip down to
+    the block boundary, quantised keys with the clamped query below it."""
+    from vqtree_amd.ops import attn_vq as A
+
+    print("fullsize: reference-shaped route, 4 heads, 8192 tokens, window 1024, 512 codewords", flush=True)
+    B, H, N, D, W, C = 1, 4, 8192, 128, 1024, 512
+    g = torch.Generator(device="cuda").manual_seed(9)
+    q, k, v = (torch.randn(B, H, N, D, generator=g, device="cuda").bfloat16() for _ in range(3))
+    cb = torch.randn(H, C, D, generator=g, device="cuda").bfloat16()
+    pos = torch.arange(N, device="cuda").unsqueeze(0)
+    cache = A.VectorQuantizedReRoPECache(W, cb)
+    out = A.dispatch_attn(q, k, v, pos, cache).view(B, N, H, D)
+    torch.cuda.synchronize()
+    q1, k1, q2 = A.rerope_operands(q, k, pos, W)
+    ids = cache.key_codes[0][..., 0].long().cpu() if cache.key_codes else None
+    if ids is None:  # more than 256 codewords: the cache keeps no uint8 codes; encode again
+        from vqtree_amd.ops.mini_vq import quantize_ids
+        ids = quantize_ids(k, cb).cpu()
+    scale = 1.0 / math.sqrt(D)
+    for h in (0, 3):
+        k_hat = cb[h].float().cpu()[ids[0, h]]  # [N,D]
+        q1h, q2h, k1h, kh, vh = (x[0, h].float().cpu() for x in (q1, q2, k1, k, v))
+        for i in (0, 1000, W + 127, W + 128, 3000, 5555, N - 1):
+            boundary = max(0, (i - W) // 128 * 128)
+            local = max(0, i - W)
+            s = torch.cat([k_hat[:boundary] @ q2h[i], kh[boundary:local] @ q2h[i], k1h[local:i + 1] @ q1h[i]]) * scale
+            want = torch.softmax(s, 0) @ vh[:i + 1]
+            assert_close_16(out[0, i, h].cpu(), want, f"head {h} row {i}")
