@@ -209,6 +209,20 @@ int vqa_merge_state_inplace_bf16(void* o, float* s, const void* o_other, const f
 int vqa_merge_state_inplace_f16(void* o, float* s, const void* o_other, const float* s_other, int B, int H, int N,
                                 int D, const int64_t* strides, vqa_stream_t stream);
 
+/* vqa_decode with the number of keys read from device memory when the kernels run: *n_keys_dev (clamped to
+ * [0, N_max]) keys are attended, N_max is the bound the buffers, the workspace and the split count are sized for.  One
+ * recorded launch sequence (a HIP graph of a decode step) can then be replayed while the cache grows.  No counterpart
+ * in the reference (its decode route is not functional, ops/attn_vq.py:445-479). */
+int vqa_decode_devlen_bf16(const void* q, const uint8_t* codes, const void* codebooks, const void* v, void* out,
+                           float* lse, void* workspace, size_t workspace_bytes, int B, int H, int N_max, int D, int M,
+                           int K, const int64_t* strides, float sm_scale, int num_splits, const int32_t* n_keys_dev,
+                           vqa_stream_t stream);
+
+int vqa_decode_devlen_f16(const void* q, const uint8_t* codes, const void* codebooks, const void* v, void* out,
+                          float* lse, void* workspace, size_t workspace_bytes, int B, int H, int N_max, int D, int M,
+                          int K, const int64_t* strides, float sm_scale, int num_splits, const int32_t* n_keys_dev,
+                          vqa_stream_t stream);
+
 /* ------------------------------------------------------------------------------------------------------------------
  * seqlen_q = 1 attention over exact keys: out[b,h] = softmax_j(sm_scale * <q[b,h], k[b,h,j]>) . v[b,h,j], no mask.
  * The generation step of the ReRoPE module and the short-context fallback of the VQ module make this call through a

@@ -145,3 +145,48 @@ def test_hybrid_decode_state_merge():
     scores = case.q.float().cpu() @ keys.transpose(-1, -2) * case.softmax_scale
     want, _ = oracle.attend(scores, torch.ones(1, N, dtype=torch.bool), case.v.float().cpu())
     assert_close_16(merged.cpu(), want, "hybrid decode")
+
+
+def test_decode_with_device_side_key_count_and_graph_replay():
+    """The key count read from device memory equals slicing the cache on the host, eagerly and inside a HIP graph that
+    is recorded once and replayed for growing counts (with eager work and synchronisations between the replays)."""
+    B, H, N_max, D, M = 2, 4, 3000, 128, 4
+    case = decode_case(B, H, N_max, D, M, device="cuda", seed=31)
+    n_dev = torch.zeros(1, dtype=torch.int32, device="cuda")
+    lib_splits = 6
+    counts = [1, 63, 64, 257, 1024, 2999, 3000]
+    eager = {}
+    for n in counts:
+        eager[n] = attn_vq_decode(case.q, case.codes[:, :, :n], case.codebooks, case.v[:, :, :n], num_splits=lib_splits)
+        n_dev.fill_(n)
+        got = attn_vq_decode(case.q, case.codes, case.codebooks, case.v, num_splits=lib_splits, n_keys=n_dev)
+        assert_close_16(got.cpu(), eager[n].float().cpu(), f"device-side count {n}")
+    # a count beyond the capacity is clamped; zero keys give a zero row
+    n_dev.fill_(10 ** 6)
+    assert torch.equal(attn_vq_decode(case.q, case.codes, case.codebooks, case.v, num_splits=lib_splits, n_keys=n_dev),
+                       attn_vq_decode(case.q, case.codes, case.codebooks, case.v, num_splits=lib_splits))
+    n_dev.fill_(0)
+    assert not attn_vq_decode(case.q, case.codes, case.codebooks, case.v, num_splits=lib_splits, n_keys=n_dev).any()
+
+    from vqtree_amd import _lib
+    out = torch.empty_like(case.q)
+    ws = torch.empty(_lib.load().vqa_decode_workspace_bytes(B, H, N_max, D, M, 256, lib_splits), dtype=torch.uint8,
+                     device="cuda")
+    n_dev.fill_(counts[0])
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):  # warm-up on the capture stream before recording
+        attn_vq_decode(case.q, case.codes, case.codebooks, case.v, num_splits=lib_splits, n_keys=n_dev, out=out,
+                       workspace=ws)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        attn_vq_decode(case.q, case.codes, case.codebooks, case.v, num_splits=lib_splits, n_keys=n_dev, out=out,
+                       workspace=ws)
+    for round_ in range(2):
+        for n in counts:
+            n_dev.fill_(n)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert_close_16(out.cpu(), eager[n].float().cpu(), f"graph replay, count {n}, round {round_}")
+            _ = (case.v[:, :, :64].float().sum(), torch.cuda.synchronize())  # unrelated eager work between replays

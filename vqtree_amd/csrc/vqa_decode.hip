@@ -121,7 +121,8 @@ __global__ __launch_bounds__(kThreads, 3) void main_kernel(const uint8_t* __rest
                                                            const uint16_t* __restrict__ v,
                                                            const float* __restrict__ lut,
                                                            float* __restrict__ part_o, float* __restrict__ part_ml,
-                                                           int H, int N, int S, int keys_per_split, Strides st) {
+                                                           int H, int N, int S, int keys_per_split, Strides st,
+                                                           const int* __restrict__ n_keys_dev) {
     constexpr int LPR = D / 8;
     constexpr int G = kWave / LPR;
     constexpr int R = kBatch / G;
@@ -141,6 +142,12 @@ __global__ __launch_bounds__(kThreads, 3) void main_kernel(const uint8_t* __rest
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int g = lane / LPR, c = lane % LPR;
+    if (n_keys_dev != nullptr) {
+        // the number of keys lives in device memory (a launch recorded once and replayed as the cache grows):
+        // N is only the bound the buffers were sized for
+        N = max(0, min(N, *n_keys_dev));
+        keys_per_split = ((N + S - 1) / S + kThreads - 1) / kThreads * kThreads;
+    }
 
     for (int i = tid; i < M * kLutStride; i += kThreads) s_lut[i] = lut[(int64_t)bh * M * kLutStride + i];
     __syncthreads();
@@ -508,16 +515,16 @@ inline int default_splits(int B, int H, int N) {
 
 template <typename Tag, int D, int M>
 int launch_main(const uint8_t* codes, const uint16_t* v, const float* lut, float* po, float* pml, int B, int H, int N,
-                int S, int kps, const Strides& st, hipStream_t stream) {
+                int S, int kps, const Strides& st, const int* n_keys_dev, hipStream_t stream) {
     hipLaunchKernelGGL((main_kernel<Tag, D, M>), dim3(S, B * H), dim3(kThreads), 0, stream, codes, v, lut, po, pml, H,
-                       N, S, kps, st);
+                       N, S, kps, st, n_keys_dev);
     return launch_status();
 }
 
 template <typename Tag, int D>
 int run_d(const void* q, const uint8_t* codes, const void* codebooks, const void* v, void* out, float* lse,
           void* workspace, int B, int H, int N, int M, int K, const Strides& st, float sm_scale, int S,
-          hipStream_t stream) {
+          const int* n_keys_dev, hipStream_t stream) {
     const Workspace ws = plan(B, H, D, M, S);
     char* base = static_cast<char*>(workspace);
     float* lut = reinterpret_cast<float*>(base + ws.lut_off);
@@ -537,10 +544,10 @@ int run_d(const void* q, const uint8_t* codes, const void* codebooks, const void
     int kps = (N + S - 1) / S;
     kps = (kps + kThreads - 1) / kThreads * kThreads;
     switch (M) {
-        case 1: rc = launch_main<Tag, D, 1>(codes, v16, lut, po, pml, B, H, N, S, kps, st, stream); break;
-        case 2: rc = launch_main<Tag, D, 2>(codes, v16, lut, po, pml, B, H, N, S, kps, st, stream); break;
-        case 4: rc = launch_main<Tag, D, 4>(codes, v16, lut, po, pml, B, H, N, S, kps, st, stream); break;
-        case 8: rc = launch_main<Tag, D, 8>(codes, v16, lut, po, pml, B, H, N, S, kps, st, stream); break;
+        case 1: rc = launch_main<Tag, D, 1>(codes, v16, lut, po, pml, B, H, N, S, kps, st, n_keys_dev, stream); break;
+        case 2: rc = launch_main<Tag, D, 2>(codes, v16, lut, po, pml, B, H, N, S, kps, st, n_keys_dev, stream); break;
+        case 4: rc = launch_main<Tag, D, 4>(codes, v16, lut, po, pml, B, H, N, S, kps, st, n_keys_dev, stream); break;
+        case 8: rc = launch_main<Tag, D, 8>(codes, v16, lut, po, pml, B, H, N, S, kps, st, n_keys_dev, stream); break;
         default: return VQA_ERR_UNSUPPORTED_CODEBOOK;
     }
     if (rc != VQA_OK) return rc;
@@ -552,7 +559,7 @@ int run_d(const void* q, const uint8_t* codes, const void* codebooks, const void
 template <typename Tag>
 int run(const void* q, const uint8_t* codes, const void* codebooks, const void* v, void* out, float* lse,
         void* workspace, size_t workspace_bytes, int B, int H, int N, int D, int M, int K, const int64_t* strides,
-        float sm_scale, int num_splits, hipStream_t stream) {
+        float sm_scale, int num_splits, const int* n_keys_dev, hipStream_t stream) {
     if (!q || !codes || !codebooks || !v || !out || !workspace || !strides) return VQA_ERR_NULL_POINTER;
     if (B <= 0 || H <= 0 || N <= 0) return VQA_ERR_BAD_SHAPE;
     if (D != 64 && D != 128) return VQA_ERR_UNSUPPORTED_HEAD_DIM;
@@ -572,8 +579,10 @@ int run(const void* q, const uint8_t* codes, const void* codebooks, const void* 
     if (S > 65535 || (int64_t)B * H > 65535) return VQA_ERR_BAD_ARGUMENT;
     if (workspace_bytes < plan(B, H, D, M, S).total) return VQA_ERR_WORKSPACE_TOO_SMALL;
     if (D == 64)
-        return run_d<Tag, 64>(q, codes, codebooks, v, out, lse, workspace, B, H, N, M, K, st, sm_scale, S, stream);
-    return run_d<Tag, 128>(q, codes, codebooks, v, out, lse, workspace, B, H, N, M, K, st, sm_scale, S, stream);
+        return run_d<Tag, 64>(q, codes, codebooks, v, out, lse, workspace, B, H, N, M, K, st, sm_scale, S, n_keys_dev,
+                              stream);
+    return run_d<Tag, 128>(q, codes, codebooks, v, out, lse, workspace, B, H, N, M, K, st, sm_scale, S, n_keys_dev,
+                           stream);
 }
 
 // strides: q(b,h) k(b,h,n) v(b,h,n) out(b,h)
@@ -660,14 +669,32 @@ int vqa_decode_bf16(const void* q, const uint8_t* codes, const void* codebooks, 
                     void* workspace, size_t workspace_bytes, int B, int H, int N, int D, int M, int K,
                     const int64_t* strides, float sm_scale, int num_splits, vqa_stream_t stream) {
     return vqa::decode::run<vqa::bf16_tag>(q, codes, codebooks, v, out, lse, workspace, workspace_bytes, B, H, N, D, M,
-                                           K, strides, sm_scale, num_splits, stream);
+                                           K, strides, sm_scale, num_splits, nullptr, stream);
 }
 
 int vqa_decode_f16(const void* q, const uint8_t* codes, const void* codebooks, const void* v, void* out, float* lse,
                    void* workspace, size_t workspace_bytes, int B, int H, int N, int D, int M, int K,
                    const int64_t* strides, float sm_scale, int num_splits, vqa_stream_t stream) {
     return vqa::decode::run<vqa::f16_tag>(q, codes, codebooks, v, out, lse, workspace, workspace_bytes, B, H, N, D, M,
-                                          K, strides, sm_scale, num_splits, stream);
+                                          K, strides, sm_scale, num_splits, nullptr, stream);
+}
+
+int vqa_decode_devlen_bf16(const void* q, const uint8_t* codes, const void* codebooks, const void* v, void* out,
+                           float* lse, void* workspace, size_t workspace_bytes, int B, int H, int N_max, int D, int M,
+                           int K, const int64_t* strides, float sm_scale, int num_splits, const int32_t* n_keys_dev,
+                           vqa_stream_t stream) {
+    if (!n_keys_dev) return VQA_ERR_NULL_POINTER;
+    return vqa::decode::run<vqa::bf16_tag>(q, codes, codebooks, v, out, lse, workspace, workspace_bytes, B, H, N_max, D,
+                                           M, K, strides, sm_scale, num_splits, n_keys_dev, stream);
+}
+
+int vqa_decode_devlen_f16(const void* q, const uint8_t* codes, const void* codebooks, const void* v, void* out,
+                          float* lse, void* workspace, size_t workspace_bytes, int B, int H, int N_max, int D, int M,
+                          int K, const int64_t* strides, float sm_scale, int num_splits, const int32_t* n_keys_dev,
+                          vqa_stream_t stream) {
+    if (!n_keys_dev) return VQA_ERR_NULL_POINTER;
+    return vqa::decode::run<vqa::f16_tag>(q, codes, codebooks, v, out, lse, workspace, workspace_bytes, B, H, N_max, D,
+                                          M, K, strides, sm_scale, num_splits, n_keys_dev, stream);
 }
 
 }  // extern "C"

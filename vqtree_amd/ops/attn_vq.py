@@ -21,11 +21,16 @@ def _last_dim_contiguous(x):
     return x if x.stride(-1) == 1 else x.contiguous()
 
 
-def attn_vq_decode(q, k_codes, codebooks, v, *, softmax_scale=None, return_lse=False, num_splits=0):
+def attn_vq_decode(q, k_codes, codebooks, v, *, softmax_scale=None, return_lse=False, num_splits=0, n_keys=None,
+                   out=None, workspace=None):
     """out[b,h] = softmax_j(scale * sum_m <q[b,h], codebooks[h,m,k_codes[b,h,j,m]]>) @ v[b,h]   (no mask).
 
     q [B,H,1,D] bf16/f16, k_codes [B,H,N,M] uint8, codebooks [H,M,K,D], v [B,H,N,D]  ->  out [B,H,1,D] (q's dtype)
     and, with return_lse, the base-2 log-sum-exp [B,H,1] fp32.
+
+    `n_keys` (int32 tensor with one element, on the device): the number of keys to attend is read from it when the
+    kernels run, N being only the capacity of the buffers -- for launch sequences recorded once (a HIP graph of a decode
+    step) and replayed as the cache grows.  `out` / `workspace` let such a caller provide the buffers.
     """
     lib = _lib.load()
     _lib.require_gpu(q, k_codes, codebooks, v)
@@ -43,11 +48,15 @@ def attn_vq_decode(q, k_codes, codebooks, v, *, softmax_scale=None, return_lse=F
         k_codes = k_codes.contiguous()
     softmax_scale = softmax_scale or 1.0 / math.sqrt(D)
 
-    out = torch.empty((B, H, 1, D), dtype=q.dtype, device=q.device)
+    if out is None:
+        out = torch.empty((B, H, 1, D), dtype=q.dtype, device=q.device)
+    assert out.shape == (B, H, 1, D) and out.dtype == q.dtype and out.stride(-1) == 1
     lse = torch.empty((B, H, 1), dtype=torch.float32, device=q.device) if return_lse else None
     splits = num_splits if num_splits > 0 else lib.vqa_decode_default_splits(B, H, N)
     ws_bytes = lib.vqa_decode_workspace_bytes(B, H, N, D, M, K, splits)
-    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
+    if workspace is None:
+        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
+    assert workspace.numel() >= ws_bytes and workspace.dtype == torch.uint8
     strides = _lib.strides_array(
         q.stride(0), q.stride(1),
         k_codes.stride(0), k_codes.stride(1),
@@ -56,15 +65,16 @@ def attn_vq_decode(q, k_codes, codebooks, v, *, softmax_scale=None, return_lse=F
         out.stride(0), out.stride(1),
     )  # fmt: skip
     with torch.cuda.device(q.device):
-        fn = getattr(lib, "vqa_decode_" + _SUFFIX[q.dtype])
-        _lib.check(
-            fn(
-                q.data_ptr(), k_codes.data_ptr(), codebooks.data_ptr(), v.data_ptr(), out.data_ptr(),
+        args = (q.data_ptr(), k_codes.data_ptr(), codebooks.data_ptr(), v.data_ptr(), out.data_ptr(),
                 lse.data_ptr() if return_lse else None,
-                workspace.data_ptr(), ws_bytes, B, H, N, D, M, K, strides, softmax_scale, splits,
-                _lib.current_stream(q.device),
-            )
-        )  # fmt: skip
+                workspace.data_ptr(), ws_bytes, B, H, N, D, M, K, strides, softmax_scale, splits)  # fmt: skip
+        if n_keys is None:
+            rc = getattr(lib, "vqa_decode_" + _SUFFIX[q.dtype])(*args, _lib.current_stream(q.device))
+        else:
+            assert n_keys.dtype == torch.int32 and n_keys.numel() == 1 and n_keys.is_cuda
+            rc = getattr(lib, "vqa_decode_devlen_" + _SUFFIX[q.dtype])(*args, n_keys.data_ptr(),
+                                                                       _lib.current_stream(q.device))
+        _lib.check(rc)
     return (out, lse) if return_lse else out
 
 
