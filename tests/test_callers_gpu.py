@@ -161,6 +161,32 @@ def test_decode_harness_with_exact_window_matches_dense_reference():
     assert (lc.float() - ld.float()).abs().max() <= 2e-2 * max(1.0, float(ld.float().abs().max()))
 
 
+def test_decode_harness_recorded_step_matches_eager_steps():
+    """The decode step recorded once as a HIP graph (cache position and key count in device memory) and replayed,
+    against the eager step on a twin model: same tokens, logits within tolerance, same appended codes."""
+    from vqtree_amd.decode_harness import VQDecodeModel
+
+    kw = dict(layers=2, hidden=256, heads=2, head_dim=128, ffn=512, vocab=1000, n_codebooks=4, window=128,
+              capacity=400, batch=2)
+    a, b = VQDecodeModel(**kw), VQDecodeModel(**kw)
+    a.fill_random_context(300), b.fill_random_context(300)
+    tok = torch.tensor([3, 777], device="cuda")
+    with torch.no_grad():
+        b.record_step(tok)  # runs one (warm-up) step eagerly on a side stream, then records
+        ta, la = a.step(tok, return_logits=True)
+        assert torch.equal(ta, b.tok) and b.length == a.length == 301
+        for step in range(6):
+            ta, la = a.step(ta, return_logits=True)
+            tb = b.replay_step()
+            torch.cuda.synchronize()
+            assert (la.float() - b.logits.float()).abs().max() <= 2e-2 * max(1.0, float(la.float().abs().max())), step
+            assert torch.equal(ta, tb), step
+            n = a.length - 1
+            assert torch.equal(a.layers[0]["codes"][:, :, n], b.layers[0]["codes"][:, :, n])
+            _ = (a.layers[1]["values"][:, :, :8].float().sum(), torch.cuda.synchronize())  # eager work between replays
+    assert b.length == a.length == 307
+
+
 def test_rerope_caller_routes():
     """Attention core of the ReRoPE module: long prefill through the full ReRoPE kernel against the dense oracle,
     cache contents after it, a short prefill (plain causal) and a generation step against dense softmax over the

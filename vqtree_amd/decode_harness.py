@@ -133,6 +133,69 @@ class VQDecodeModel:
         logits = self._rms(x) @ self.lm_head
         return (logits.argmax(-1), logits) if return_logits else logits.argmax(-1)
 
+    # ---------------------------------------------------------------------------------------------------------
+    # the same step with every position-dependent quantity in device memory, so that it can be recorded once as a
+    # HIP graph and replayed: cache writes by index_copy_ at `pos_dev`, attention over `n_dev` keys of the full
+    # buffers, the next token kept in a static buffer
+    # ---------------------------------------------------------------------------------------------------------
+    def _init_device_state(self, tokens):
+        from . import _lib
+
+        assert not self.exact_window, "the recorded step codes every key"
+        dev = self.device
+        self.tok = tokens.clone()
+        self.pos_dev = torch.tensor([self.length], dtype=torch.int64, device=dev)
+        self.n_dev = torch.tensor([self.length + 1], dtype=torch.int32, device=dev)
+        lib = _lib.load()
+        self.splits = lib.vqa_decode_default_splits(self.B, self.H, self.capacity)
+        self.ws = torch.empty(lib.vqa_decode_workspace_bytes(self.B, self.H, self.capacity, self.D, self.M, 256,
+                                                             self.splits), dtype=torch.uint8, device=dev)
+        self.attn_out = torch.empty(self.B, self.H, 1, self.D, dtype=self.dtype, device=dev)
+        self.logits = None
+
+    def _device_step(self):
+        B, H, D = self.B, self.H, self.D
+        x = self.embed[self.tok]
+        for layer in self.layers:
+            h = self._rms(x)
+            qkv = (h @ layer["wqkv"]).view(B, 3, H, D)
+            q, k, v = qkv[:, 0], qkv[:, 1], qkv[:, 2]
+            q2 = (q * self.cos_w + rotate_half(q) * self.sin_w).unsqueeze(2)
+            layer["codes"].index_copy_(2, self.pos_dev, encode_residual(k.unsqueeze(2), layer["codebooks"]))
+            layer["values"].index_copy_(2, self.pos_dev, v.unsqueeze(2))
+            attn_vq_decode(q2, layer["codes"], layer["codebooks"], layer["values"], softmax_scale=1.0 / math.sqrt(D),
+                           num_splits=self.splits, n_keys=self.n_dev, out=self.attn_out, workspace=self.ws)
+            x = x + self.attn_out.reshape(B, H * D) @ layer["wo"]
+            h = self._rms(x)
+            gate, up = (h @ layer["w_gate_up"]).chunk(2, dim=-1)
+            x = x + (torch.nn.functional.silu(gate) * up) @ layer["w_down"]
+        logits = self._rms(x) @ self.lm_head
+        self.tok.copy_(logits.argmax(-1))
+        self.pos_dev += 1
+        self.n_dev += 1
+        return logits
+
+    def record_step(self, tokens):
+        """Record one decode step as a HIP graph (after one warm-up step on a side stream, which already advances the
+        cache by one token).  `replay_step()` then runs a step per call; `self.tok` holds the newest tokens and
+        `self.logits` the logits of the last replayed step."""
+        self._init_device_state(tokens)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            self._device_step()
+        torch.cuda.current_stream().wait_stream(side)
+        self.length += 1
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            self.logits = self._device_step()
+        return self
+
+    def replay_step(self):
+        self.graph.replay()
+        self.length += 1
+        return self.tok
+
     def attention_bytes_per_step(self):
         """Algorithmic bytes of the attention path per token step: per layer codes of the coded keys + V + exact
         window keys + codebooks + q/out."""
@@ -145,12 +208,34 @@ class VQDecodeModel:
 
 
 def run(layers=32, hidden=4096, heads=32, head_dim=128, ffn=11008, vocab=32000, n_codebooks=4, context=65536, batch=4,
-        steps=128, warmup=4, window=1024, exact_window=0, device="cuda"):
-    model = VQDecodeModel(layers, hidden, heads, head_dim, ffn, vocab, n_codebooks, window, context + steps + warmup,
-                          batch, device=device, exact_window=exact_window)
+        steps=128, warmup=4, window=1024, exact_window=0, graph=0, device="cuda"):
+    model = VQDecodeModel(layers, hidden, heads, head_dim, ffn, vocab, n_codebooks, window,
+                          context + steps + warmup + 2, batch, device=device, exact_window=exact_window)
     model.fill_random_context(context)
     g = torch.Generator(device=device).manual_seed(7)
     tokens = torch.randint(0, vocab, (batch,), generator=g, device=device)
+    if graph:
+        with torch.no_grad():
+            model.record_step(tokens)
+            for _ in range(warmup):
+                model.replay_step()
+            torch.cuda.synchronize()
+            bytes_mid = None
+            t0 = time.perf_counter()
+            for s in range(steps):
+                if s == steps // 2:
+                    bytes_mid = model.attention_bytes_per_step()
+                model.replay_step()
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+        return {
+            "workload": f"{layers}-layer Llama-2-7B-shaped greedy decode, batch {batch}, context {context}, VQ key "
+                        f"cache {n_codebooks}x256 per layer, {steps} steps, one HIP graph replay per step",
+            "us_per_step": round(dt / steps * 1e6, 1),
+            "attention_bytes_per_step": bytes_mid,
+            "note": "whole-step wall time; the step (projections, MLP, key encoder, cache append, attention) is "
+                    "recorded once with the cache position and key count in device memory",
+        }
     with torch.no_grad():
         for _ in range(warmup):
             tokens = model.step(tokens)
@@ -183,6 +268,6 @@ def run(layers=32, hidden=4096, heads=32, head_dim=128, ffn=11008, vocab=32000, 
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     for name, default in (("layers", 32), ("context", 65536), ("batch", 4), ("steps", 128), ("warmup", 4),
-                          ("exact_window", 0)):
+                          ("exact_window", 0), ("graph", 0)):
         ap.add_argument("--" + name, type=int, default=default)
     print(json.dumps(run(**vars(ap.parse_args()))))
