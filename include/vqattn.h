@@ -245,6 +245,30 @@ int vqa_decode_exact_f16(const void* q, const void* k, const void* v, void* out,
                          int num_splits, vqa_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------------------------------
+ * seqlen_q = 1 attention with an exact recent window: keys [0, N - W) are scored through their codes with q_far (the
+ * position-clamped query of the ReRoPE VQ module), the last W keys exactly with q_win against k_win [B,H,W,D]; v
+ * [B,H,N,D] covers both ranges.  The coded and the exact streaming kernels write their split states into one
+ * workspace and one merge produces out / lse.  This is the decode-time counterpart of the cache the reference
+ * describes (codes for the far context, a window of exact keys: ops/attn_vq.py:31-52, 290-333), which it never got
+ * to run at seqlen_q == 1.
+ *   strides[0..16] = q_far(b,h) q_win(b,h) codes(b,h) codebooks(h,m,k) v(b,h,n) k_win(b,h,n) out(b,h).
+ *   codes may be null when W == N.  Workspace: vqa_decode_windowed_workspace_bytes, 256-byte aligned.
+ * ------------------------------------------------------------------------------------------------------------------ */
+#define VQA_DECODE_WINDOWED_NUM_STRIDES 17
+
+size_t vqa_decode_windowed_workspace_bytes(int B, int H, int N, int W, int D, int M);
+
+int vqa_decode_windowed_bf16(const void* q_far, const void* q_win, const uint8_t* codes, const void* codebooks,
+                             const void* v, const void* k_win, void* out, float* lse, void* workspace,
+                             size_t workspace_bytes, int B, int H, int N, int W, int D, int M, int K,
+                             const int64_t* strides, float sm_scale, vqa_stream_t stream);
+
+int vqa_decode_windowed_f16(const void* q_far, const void* q_win, const uint8_t* codes, const void* codebooks,
+                            const void* v, const void* k_win, void* out, float* lse, void* workspace,
+                            size_t workspace_bytes, int B, int H, int N, int W, int D, int M, int K,
+                            const int64_t* strides, float sm_scale, vqa_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------------------------------
  * Key encoder: nearest-codeword search of every key against its head's codebooks.
  *   mode 0: id_m = argmax_c <x, codebooks[h,m,c]> for every codebook m independently (inner product, first maximum
  *           on ties) -- replaces multi_head_single_quantize, ops/mini_vq.py:4-18 (M = 1); with round_scores != 0 the

@@ -124,3 +124,18 @@ def test_exact_decode_rejects_bad_arguments_before_any_launch(lib):
     assert call(D=96) == -3
     assert call(v=24) == -5 and call(ws=64) == -5
     assert call(ws_bytes=need - 1) == -6
+
+
+def test_windowed_decode_rejects_bad_arguments_before_any_launch(lib):
+    s17 = _lib.strides_array(*([8] * 17))
+    need = lib.vqa_decode_windowed_workspace_bytes(2, 4, 5000, 512, 128, 4)
+    assert need > lib.vqa_decode_workspace_bytes(2, 4, 5000 - 512, 128, 4, 256, 0) and need % 256 == 0
+    assert lib.vqa_decode_windowed_workspace_bytes(2, 4, 100, 200, 128, 4) == 0  # window longer than the cache
+    call = lambda qf=16, qw=16, codes=16, cb=16, v=16, kw=16, out=16, ws=256, ws_bytes=1 << 24, N=5000, W=512, D=128, M=4: \
+        lib.vqa_decode_windowed_bf16(qf, qw, codes, cb, v, kw, out, None, ws, ws_bytes, 2, 4, N, W, D, M, 256, s17, 1.0,
+                                     None)
+    assert call(qw=None) == -1 and call(kw=None) == -1 and call(codes=None) == -1
+    assert call(W=0) == -2 and call(W=6000) == -2
+    assert call(D=96) == -3 and call(M=3) == -4
+    assert call(kw=24) == -5
+    assert call(ws_bytes=need - 1) == -6

@@ -139,12 +139,26 @@ def test_hybrid_decode_state_merge():
     g = torch.Generator("cpu").manual_seed(23)
     k_win = torch.randn(B, H, W, D, generator=g).bfloat16().cuda()
     far = N - W
-    merged = attn_vq_decode_windowed(case.q, case.codes, case.codebooks, case.v, k_win)
+    merged, lse = attn_vq_decode_windowed(case.q, case.codes, case.codebooks, case.v, k_win, return_lse=True)
     k_hat = oracle.reconstruct_keys(case.codes[:, :, :far].cpu(), case.codebooks.cpu())
     keys = torch.cat([k_hat, k_win.float().cpu()], dim=2)
     scores = case.q.float().cpu() @ keys.transpose(-1, -2) * case.softmax_scale
-    want, _ = oracle.attend(scores, torch.ones(1, N, dtype=torch.bool), case.v.float().cpu())
+    want, want_lse = oracle.attend(scores, torch.ones(1, N, dtype=torch.bool), case.v.float().cpu())
     assert_close_16(merged.cpu(), want, "hybrid decode")
+    assert_close_lse(lse.cpu()[..., 0], want_lse[..., 0], atol=1e-2)
+    # the window may cover everything (no coded keys), and may use its own query
+    g2 = torch.Generator("cpu").manual_seed(24)
+    k_all = torch.randn(B, H, N, D, generator=g2).bfloat16().cuda()
+    q_w = torch.randn(B, H, 1, D, generator=g2).bfloat16().cuda()
+    full = attn_vq_decode_windowed(case.q, case.codes, case.codebooks, case.v, k_all, q_window=q_w)
+    sc = q_w.float().cpu() @ k_all.float().cpu().transpose(-1, -2) * case.softmax_scale
+    want_full, _ = oracle.attend(sc, torch.ones(1, N, dtype=torch.bool), case.v.float().cpu())
+    assert_close_16(full.cpu(), want_full, "window covers every key")
+    mixed = attn_vq_decode_windowed(case.q, case.codes, case.codebooks, case.v, k_win, q_window=q_w)
+    s_mixed = torch.cat([case.q.float().cpu() @ k_hat.transpose(-1, -2),
+                         q_w.float().cpu() @ k_win.float().cpu().transpose(-1, -2)], dim=-1) * case.softmax_scale
+    want_mixed, _ = oracle.attend(s_mixed, torch.ones(1, N, dtype=torch.bool), case.v.float().cpu())
+    assert_close_16(mixed.cpu(), want_mixed, "separate window query")
 
 
 def test_decode_with_device_side_key_count_and_graph_replay():

@@ -122,7 +122,8 @@ __global__ __launch_bounds__(kThreads, 3) void main_kernel(const uint8_t* __rest
                                                            const float* __restrict__ lut,
                                                            float* __restrict__ part_o, float* __restrict__ part_ml,
                                                            int H, int N, int S, int keys_per_split, Strides st,
-                                                           const int* __restrict__ n_keys_dev) {
+                                                           const int* __restrict__ n_keys_dev, int slot_stride,
+                                                           int slot_off) {
     constexpr int LPR = D / 8;
     constexpr int G = kWave / LPR;
     constexpr int R = kBatch / G;
@@ -275,7 +276,8 @@ __global__ __launch_bounds__(kThreads, 3) void main_kernel(const uint8_t* __rest
             o += wgt * t;
             l += wgt * s_l[w];
         }
-        const int64_t slot = (int64_t)bh * S + split;
+        // partial states of one (batch, head) are contiguous: slot_stride of them, this launch's from slot_off on
+        const int64_t slot = (int64_t)bh * slot_stride + slot_off + split;
         part_o[slot * D + tid] = o;
         if (tid == 0) {
             part_ml[slot * 2] = m_all;
@@ -328,7 +330,7 @@ __global__ __launch_bounds__(kThreads, 2) void exact_kernel(const uint16_t* __re
                                                             const uint16_t* __restrict__ v,
                                                             float* __restrict__ part_o, float* __restrict__ part_ml,
                                                             int H, int N, int S, int keys_per_split, ExactStrides st,
-                                                            float scale_log2e) {
+                                                            float scale_log2e, int slot_stride, int slot_off) {
     constexpr int LPR = D / 8;
     constexpr int G = kWave / LPR;
     constexpr int R = kBatch / G;
@@ -476,7 +478,8 @@ __global__ __launch_bounds__(kThreads, 2) void exact_kernel(const uint16_t* __re
             o += wgt * t;
             l += wgt * s_l[w];
         }
-        const int64_t slot = (int64_t)bh * S + split;
+        // partial states of one (batch, head) are contiguous: slot_stride of them, this launch's from slot_off on
+        const int64_t slot = (int64_t)bh * slot_stride + slot_off + split;
         part_o[slot * D + tid] = o;
         if (tid == 0) {
             part_ml[slot * 2] = m_all;
@@ -515,9 +518,10 @@ inline int default_splits(int B, int H, int N) {
 
 template <typename Tag, int D, int M>
 int launch_main(const uint8_t* codes, const uint16_t* v, const float* lut, float* po, float* pml, int B, int H, int N,
-                int S, int kps, const Strides& st, const int* n_keys_dev, hipStream_t stream) {
+                int S, int kps, const Strides& st, const int* n_keys_dev, int slot_stride, int slot_off,
+                hipStream_t stream) {
     hipLaunchKernelGGL((main_kernel<Tag, D, M>), dim3(S, B * H), dim3(kThreads), 0, stream, codes, v, lut, po, pml, H,
-                       N, S, kps, st, n_keys_dev);
+                       N, S, kps, st, n_keys_dev, slot_stride, slot_off);
     return launch_status();
 }
 
@@ -544,10 +548,10 @@ int run_d(const void* q, const uint8_t* codes, const void* codebooks, const void
     int kps = (N + S - 1) / S;
     kps = (kps + kThreads - 1) / kThreads * kThreads;
     switch (M) {
-        case 1: rc = launch_main<Tag, D, 1>(codes, v16, lut, po, pml, B, H, N, S, kps, st, n_keys_dev, stream); break;
-        case 2: rc = launch_main<Tag, D, 2>(codes, v16, lut, po, pml, B, H, N, S, kps, st, n_keys_dev, stream); break;
-        case 4: rc = launch_main<Tag, D, 4>(codes, v16, lut, po, pml, B, H, N, S, kps, st, n_keys_dev, stream); break;
-        case 8: rc = launch_main<Tag, D, 8>(codes, v16, lut, po, pml, B, H, N, S, kps, st, n_keys_dev, stream); break;
+        case 1: rc = launch_main<Tag, D, 1>(codes, v16, lut, po, pml, B, H, N, S, kps, st, n_keys_dev, S, 0, stream); break;
+        case 2: rc = launch_main<Tag, D, 2>(codes, v16, lut, po, pml, B, H, N, S, kps, st, n_keys_dev, S, 0, stream); break;
+        case 4: rc = launch_main<Tag, D, 4>(codes, v16, lut, po, pml, B, H, N, S, kps, st, n_keys_dev, S, 0, stream); break;
+        case 8: rc = launch_main<Tag, D, 8>(codes, v16, lut, po, pml, B, H, N, S, kps, st, n_keys_dev, S, 0, stream); break;
         default: return VQA_ERR_UNSUPPORTED_CODEBOOK;
     }
     if (rc != VQA_OK) return rc;
@@ -615,10 +619,10 @@ int run_exact(const void* q, const void* k, const void* v, void* out, float* lse
     const uint16_t* v16 = static_cast<const uint16_t*>(v);
     if (D == 64) {
         hipLaunchKernelGGL((exact_kernel<Tag, 64>), dim3(S, B * H), dim3(kThreads), 0, stream, q16, k16, v16, po, pml,
-                           H, N, S, kps, es, sm_scale * kLog2e);
+                           H, N, S, kps, es, sm_scale * kLog2e, S, 0);
     } else {
         hipLaunchKernelGGL((exact_kernel<Tag, 128>), dim3(S, B * H), dim3(kThreads), 0, stream, q16, k16, v16, po, pml,
-                           H, N, S, kps, es, sm_scale * kLog2e);
+                           H, N, S, kps, es, sm_scale * kLog2e, S, 0);
     }
     int rc = launch_status();
     if (rc != VQA_OK) return rc;
@@ -631,10 +635,128 @@ int run_exact(const void* q, const void* k, const void* v, void* out, float* lse
     return launch_status();
 }
 
+// Coded far keys + exact recent window in one call: keys [0, N - W) are scored through their codes with q_far, the
+// last W keys exactly (k_win [B,H,W,D]) with q_win; both streaming kernels write their split states into one
+// workspace and a single merge produces the output.
+// strides: q_far(b,h) q_win(b,h) codes(b,h) codebooks(h,m,k) v(b,h,n) k_win(b,h,n) out(b,h)
+inline void windowed_splits(int B, int H, int N, int W, int& s_far, int& s_win) {
+    s_far = N > W ? default_splits(B, H, N - W) : 0;
+    // the window is short: one workgroup step (256 keys) per split is enough to spread it over the chip
+    const int64_t bh = (int64_t)B * H;
+    int64_t s = (2048 + bh - 1) / bh;
+    const int64_t max_s = (W + kThreads - 1) / kThreads;
+    if (s > max_s) s = max_s;
+    s_win = (int)(s < 1 ? 1 : (s > 256 ? 256 : s));
+}
+
+template <typename Tag, int D>
+int run_windowed_d(const uint16_t* q_far, const uint16_t* q_win, const uint8_t* codes, const uint16_t* cb,
+                   const uint16_t* v, const uint16_t* k_win, void* out, float* lse, char* base, int B, int H, int N,
+                   int W, int M, int K, const Strides& st, const ExactStrides& es, float sm_scale, hipStream_t stream) {
+    int s_far, s_win;
+    windowed_splits(B, H, N, W, s_far, s_win);
+    const int s_tot = s_far + s_win;
+    const Workspace ws = plan(B, H, D, M, s_tot);
+    float* lut = reinterpret_cast<float*>(base + ws.lut_off);
+    float* po = reinterpret_cast<float*>(base + ws.po_off);
+    float* pml = reinterpret_cast<float*>(base + ws.pml_off);
+    int rc = VQA_OK;
+    const int far = N - W;
+    if (far > 0) {
+        const int tiles = (K + 15) / 16;
+        hipLaunchKernelGGL((lut_kernel<Tag, D>), dim3((tiles + kWaves - 1) / kWaves, H * M), dim3(kThreads), 0, stream,
+                           q_far, cb, lut, B, H, M, K, st, sm_scale * kLog2e);
+        if ((rc = launch_status()) != VQA_OK) return rc;
+        int kps = ((far + s_far - 1) / s_far + kThreads - 1) / kThreads * kThreads;
+        switch (M) {
+            case 1: rc = launch_main<Tag, D, 1>(codes, v, lut, po, pml, B, H, far, s_far, kps, st, nullptr, s_tot, 0, stream); break;
+            case 2: rc = launch_main<Tag, D, 2>(codes, v, lut, po, pml, B, H, far, s_far, kps, st, nullptr, s_tot, 0, stream); break;
+            case 4: rc = launch_main<Tag, D, 4>(codes, v, lut, po, pml, B, H, far, s_far, kps, st, nullptr, s_tot, 0, stream); break;
+            case 8: rc = launch_main<Tag, D, 8>(codes, v, lut, po, pml, B, H, far, s_far, kps, st, nullptr, s_tot, 0, stream); break;
+            default: return VQA_ERR_UNSUPPORTED_CODEBOOK;
+        }
+        if (rc != VQA_OK) return rc;
+    }
+    const int kps_w = ((W + s_win - 1) / s_win + kThreads - 1) / kThreads * kThreads;
+    hipLaunchKernelGGL((exact_kernel<Tag, D>), dim3(s_win, B * H), dim3(kThreads), 0, stream, q_win, k_win,
+                       v + (int64_t)far * st.v_n, po, pml, H, W, s_win, kps_w, es, sm_scale * kLog2e, s_tot, s_far);
+    if ((rc = launch_status()) != VQA_OK) return rc;
+    hipLaunchKernelGGL((merge_kernel<Tag, D>), dim3(B * H), dim3(D), 0, stream, po, pml, static_cast<uint16_t*>(out),
+                       lse, H, s_tot, st);
+    return launch_status();
+}
+
+template <typename Tag>
+int run_windowed(const void* q_far, const void* q_win, const uint8_t* codes, const void* codebooks, const void* v,
+                 const void* k_win, void* out, float* lse, void* workspace, size_t workspace_bytes, int B, int H, int N,
+                 int W, int D, int M, int K, const int64_t* strides, float sm_scale, hipStream_t stream) {
+    if (!q_far || !q_win || !codebooks || !v || !k_win || !out || !workspace || !strides) return VQA_ERR_NULL_POINTER;
+    if (B <= 0 || H <= 0 || N <= 0 || W <= 0 || W > N) return VQA_ERR_BAD_SHAPE;
+    if (N > W && !codes) return VQA_ERR_NULL_POINTER;
+    if (D != 64 && D != 128) return VQA_ERR_UNSUPPORTED_HEAD_DIM;
+    if ((M != 1 && M != 2 && M != 4 && M != 8) || K < 1 || K > 256) return VQA_ERR_UNSUPPORTED_CODEBOOK;
+    Strides st = {};
+    st.q_b = strides[0], st.q_h = strides[1];
+    st.c_b = strides[4], st.c_h = strides[5];
+    st.cb_h = strides[6], st.cb_m = strides[7], st.cb_k = strides[8];
+    st.v_b = strides[9], st.v_h = strides[10], st.v_n = strides[11];
+    st.o_b = strides[15], st.o_h = strides[16];
+    ExactStrides es;
+    es.q_b = strides[2], es.q_h = strides[3];
+    es.k_b = strides[12], es.k_h = strides[13], es.k_n = strides[14];
+    es.v_b = st.v_b, es.v_h = st.v_h, es.v_n = st.v_n;
+    if (!aligned16(q_far) || !aligned16(q_win) || !aligned16(codebooks) || !aligned16(v) || !aligned16(k_win) ||
+        ((uintptr_t)workspace & 255u))
+        return VQA_ERR_MISALIGNED;
+    if ((st.q_b | st.q_h | es.q_b | es.q_h | st.cb_h | st.cb_m | st.cb_k | st.v_b | st.v_h | st.v_n | es.k_b | es.k_h |
+         es.k_n) & 7)
+        return VQA_ERR_MISALIGNED;
+    if (codes && (((uintptr_t)codes | (uintptr_t)st.c_b | (uintptr_t)st.c_h) & (uintptr_t)(M - 1)))
+        return VQA_ERR_MISALIGNED;
+    if ((int64_t)B * H > 65535) return VQA_ERR_BAD_ARGUMENT;
+    int s_far, s_win;
+    windowed_splits(B, H, N, W, s_far, s_win);
+    if (workspace_bytes < plan(B, H, D, M, s_far + s_win).total) return VQA_ERR_WORKSPACE_TOO_SMALL;
+    const uint16_t* qf = static_cast<const uint16_t*>(q_far);
+    const uint16_t* qw = static_cast<const uint16_t*>(q_win);
+    const uint16_t* cb = static_cast<const uint16_t*>(codebooks);
+    const uint16_t* v16 = static_cast<const uint16_t*>(v);
+    const uint16_t* kw = static_cast<const uint16_t*>(k_win);
+    char* base = static_cast<char*>(workspace);
+    if (D == 64)
+        return run_windowed_d<Tag, 64>(qf, qw, codes, cb, v16, kw, out, lse, base, B, H, N, W, M, K, st, es, sm_scale,
+                                       stream);
+    return run_windowed_d<Tag, 128>(qf, qw, codes, cb, v16, kw, out, lse, base, B, H, N, W, M, K, st, es, sm_scale,
+                                    stream);
+}
+
 }  // namespace decode
 }  // namespace vqa
 
 extern "C" {
+
+size_t vqa_decode_windowed_workspace_bytes(int B, int H, int N, int W, int D, int M) {
+    if (B <= 0 || H <= 0 || N <= 0 || W <= 0 || W > N || D <= 0 || M <= 0) return 0;
+    int s_far, s_win;
+    vqa::decode::windowed_splits(B, H, N, W, s_far, s_win);
+    return vqa::decode::plan(B, H, D, M, s_far + s_win).total;
+}
+
+int vqa_decode_windowed_bf16(const void* q_far, const void* q_win, const uint8_t* codes, const void* codebooks,
+                             const void* v, const void* k_win, void* out, float* lse, void* workspace,
+                             size_t workspace_bytes, int B, int H, int N, int W, int D, int M, int K,
+                             const int64_t* strides, float sm_scale, vqa_stream_t stream) {
+    return vqa::decode::run_windowed<vqa::bf16_tag>(q_far, q_win, codes, codebooks, v, k_win, out, lse, workspace,
+                                                    workspace_bytes, B, H, N, W, D, M, K, strides, sm_scale, stream);
+}
+
+int vqa_decode_windowed_f16(const void* q_far, const void* q_win, const uint8_t* codes, const void* codebooks,
+                            const void* v, const void* k_win, void* out, float* lse, void* workspace,
+                            size_t workspace_bytes, int B, int H, int N, int W, int D, int M, int K,
+                            const int64_t* strides, float sm_scale, vqa_stream_t stream) {
+    return vqa::decode::run_windowed<vqa::f16_tag>(q_far, q_win, codes, codebooks, v, k_win, out, lse, workspace,
+                                                   workspace_bytes, B, H, N, W, D, M, K, strides, sm_scale, stream);
+}
 
 size_t vqa_decode_exact_workspace_bytes(int B, int H, int N, int D, int num_splits) {
     if (B <= 0 || H <= 0 || N <= 0 || D <= 0) return 0;

@@ -19,7 +19,7 @@ import time
 
 import torch
 
-from .ops.attn_vq import attn_exact_decode, attn_vq_decode, attn_vq_decode_windowed, rope_tables, rotate_half
+from .ops.attn_vq import attn_vq_decode, attn_vq_decode_windowed, rope_tables, rotate_half
 from .ops.mini_vq import RESIDUAL, encode_keys
 
 
@@ -94,8 +94,6 @@ class VQDecodeModel:
         q_win = (q_raw * self.cos[n] + rotate_half(q_raw) * self.sin[n]).unsqueeze(2)
         if attention is not None:
             return attention(q_far, q_win, codes, layer["codebooks"], values, k_win, softmax_scale=scale)
-        if w == n + 1:
-            return attn_exact_decode(q_win, k_win, values, softmax_scale=scale)
         return attn_vq_decode_windowed(q_far, codes, layer["codebooks"], values, k_win, softmax_scale=scale,
                                        q_window=q_win)
 
@@ -261,7 +259,7 @@ def run(layers=32, hidden=4096, heads=32, head_dim=128, ffn=11008, vocab=32000, 
         "attention_GBps": round(bytes_mid / (attn_us * 1e-6) / 1e9, 1),
         "attention_hbm_frac": round(bytes_mid / (attn_us * 1e-6) / 8e12, 4),
         "note": "us_per_step is whole-step wall time (projections, MLP, key encoder, attention); attention_us_per_step "
-                "sums HIP-event intervals around the attention calls of all layers (3 kernels each; 6 with an exact window)",
+                "sums HIP-event intervals around the attention calls of all layers (3 kernels each; 4 with an exact window)",
     }
 
 

@@ -103,26 +103,42 @@ def attn_exact_decode(q, k, v, *, softmax_scale=None, return_lse=False, num_spli
     return (out, lse) if return_lse else out
 
 
-def attn_vq_decode_windowed(q, k_codes, codebooks, v, k_window, *, softmax_scale=None, q_window=None):
+def attn_vq_decode_windowed(q, k_codes, codebooks, v, k_window, *, softmax_scale=None, q_window=None,
+                            return_lse=False):
     """seqlen_q == 1 attention with an exact window: the last `k_window.shape[2]` keys are scored exactly
     (k_window [B,H,W,D], with `q_window` when the window uses another query, e.g. another rotary position), every
-    earlier key through its codes; v [B,H,N,D] covers both.  Two streaming passes over disjoint key ranges and one
-    base-2 log-sum-exp merge."""
-    from .triton_fused_vq_attn import merge_state_in_place
-
-    B, H, _, D = q.shape
-    N, W = v.shape[2], k_window.shape[2]
-    assert 0 < W <= N and k_codes.shape[2] >= N - W
+    earlier key through its codes; v [B,H,N,D] covers both.  One call: the coded and the exact streaming kernels
+    write their split states into one workspace and a single merge produces the output."""
+    lib = _lib.load()
     q_window = q if q_window is None else q_window
-    if W == N:
-        return attn_exact_decode(q_window, k_window, v, softmax_scale=softmax_scale)
-    far = N - W
-    o_far, l_far = attn_vq_decode(q, k_codes[:, :, :far], codebooks, v[:, :, :far], softmax_scale=softmax_scale,
-                                  return_lse=True)
-    o_win, l_win = attn_exact_decode(q_window, k_window, v[:, :, far:], softmax_scale=softmax_scale, return_lse=True)
-    # merge layout [rows, heads, D] / [rows, heads] with one row
-    merge_state_in_place(o_far.view(1, B * H, D), l_far.view(1, B * H), o_win.view(1, B * H, D), l_win.view(1, B * H))
-    return o_far
+    _lib.require_gpu(q, q_window, k_codes, codebooks, v, k_window)
+    B, H, one, D = q.shape
+    N, W = v.shape[2], k_window.shape[2]
+    M, K = codebooks.shape[1], codebooks.shape[2]
+    assert one == 1 and q_window.shape == q.shape and 0 < W <= N and k_codes.shape[2] >= N - W
+    assert k_window.shape == (B, H, W, D) and v.shape == (B, H, N, D) and codebooks.shape == (H, M, K, D)
+    assert q.dtype == q_window.dtype == codebooks.dtype == v.dtype == k_window.dtype and q.dtype in _SUFFIX
+    assert k_codes.dtype == torch.uint8 and k_codes.shape[3] == M
+    q, q_window, codebooks, v, k_window = map(_last_dim_contiguous, (q, q_window, codebooks, v, k_window))
+    if k_codes.stride(3) != 1 or k_codes.stride(2) != M:
+        k_codes = k_codes.contiguous()
+    softmax_scale = softmax_scale or 1.0 / math.sqrt(D)
+    out = torch.empty((B, H, 1, D), dtype=q.dtype, device=q.device)
+    lse = torch.empty((B, H, 1), dtype=torch.float32, device=q.device) if return_lse else None
+    ws = torch.empty(lib.vqa_decode_windowed_workspace_bytes(B, H, N, W, D, M), dtype=torch.uint8, device=q.device)
+    strides = _lib.strides_array(q.stride(0), q.stride(1), q_window.stride(0), q_window.stride(1),
+                                 k_codes.stride(0), k_codes.stride(1),
+                                 codebooks.stride(0), codebooks.stride(1), codebooks.stride(2),
+                                 v.stride(0), v.stride(1), v.stride(2),
+                                 k_window.stride(0), k_window.stride(1), k_window.stride(2),
+                                 out.stride(0), out.stride(1))
+    with torch.cuda.device(q.device):
+        rc = getattr(lib, "vqa_decode_windowed_" + _SUFFIX[q.dtype])(
+            q.data_ptr(), q_window.data_ptr(), k_codes.data_ptr(), codebooks.data_ptr(), v.data_ptr(),
+            k_window.data_ptr(), out.data_ptr(), None if lse is None else lse.data_ptr(), ws.data_ptr(), ws.numel(),
+            B, H, N, W, D, M, K, strides, softmax_scale, _lib.current_stream(q.device))
+    _lib.check(rc)
+    return (out, lse) if return_lse else out
 
 
 def attn_vq_prefill(q, k_codes, codebooks, v, *, k_exact=None, window_size=0, causal=True, softmax_scale=None,
