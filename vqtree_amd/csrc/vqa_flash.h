@@ -17,16 +17,6 @@
 
 #include "vqa_common.h"
 
-// wave priority while a wave issues its MFMA bursts (0 = leave the default)
-#ifndef VQA_MFMA_PRIO_LEVEL
-#define VQA_MFMA_PRIO_LEVEL 0
-#endif
-#if VQA_MFMA_PRIO_LEVEL > 0
-#define VQA_MFMA_PRIO(on) __builtin_amdgcn_s_setprio((on) ? VQA_MFMA_PRIO_LEVEL : 0)
-#else
-#define VQA_MFMA_PRIO(on) ((void)0)
-#endif
-
 namespace vqa {
 namespace flash {
 
@@ -53,8 +43,6 @@ struct Geom {
     static constexpr int kTileBytes = kBN * kRowBytes;
     static constexpr int kChunksPerRow = D / 8;                 // 16-byte chunks per row
     static constexpr int kRowsPerInstr = 64 / kChunksPerRow;    // rows one wave-wide 16-byte load covers
-    static constexpr int kRowsPerWave = kBN / kWaves;           // 16
-    static constexpr int kInstr = kRowsPerWave / kRowsPerInstr; // direct-to-LDS loads per wave and tile
     static constexpr int kRowsPerBankCycle = 256 / kRowBytes;   // rows that share one sweep over the 64 banks
     static constexpr int kKSteps = D / 16;                      // 32x32x16 steps along head_dim
     static constexpr int kDBlocks = D / 32;                     // 32-row blocks of O^T
@@ -214,14 +202,12 @@ __device__ __forceinline__ void qk_mma(f32x16_t (&s)[2], const QFrag<Tag, D>& q,
     for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
         for (int e = 0; e < 16; ++e) s[kb][e] = 0.f;
-    VQA_MFMA_PRIO(1);
 #pragma unroll
     for (int i = 0; i < kSteps; ++i) {
         if (i + kAhead < kSteps) a[(i + kAhead) % (kAhead + 1)] = frag(i + kAhead);
         s[i % 2] = Elem<Tag>::mfma32(a[i % (kAhead + 1)], q.f[i / 2], s[i % 2]);
         __builtin_amdgcn_sched_barrier(0);
     }
-    VQA_MFMA_PRIO(0);
 }
 
 // One 32-key block of S^T (key block kb of the tile), for the rarely taken multi-pair tiles where register
@@ -281,7 +267,6 @@ __device__ __forceinline__ void pv_mma(f32x16_t (&o)[Geom<D>::kDBlocks], const t
     };
 #pragma unroll
     for (int i = 0; i < kAhead; ++i) fetch(i);
-    VQA_MFMA_PRIO(1);
 #pragma unroll
     for (int i = 0; i < kSteps; ++i) {
         if (i + kAhead < kSteps) fetch(i + kAhead);
@@ -291,7 +276,6 @@ __device__ __forceinline__ void pv_mma(f32x16_t (&o)[Geom<D>::kDBlocks], const t
         o[i % DB] = Elem<Tag>::mfma32(__builtin_bit_cast(vec8, av), p[kbj >> 1][kbj & 1], o[i % DB]);
         __builtin_amdgcn_sched_barrier(0);
     }
-    VQA_MFMA_PRIO(0);
 }
 
 // Online-softmax state of one wave: every lane carries the running max of ITS query (identical in lane ^ 32) and
