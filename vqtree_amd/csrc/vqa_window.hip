@@ -388,29 +388,43 @@ __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict_
                                                       int H, int N, int M, int64_t c_sb, int64_t c_sh, int64_t cb_sh,
                                                       int64_t cb_sm, int64_t cb_sk) {
     constexpr int CPR = D / 8;
+    constexpr int KPT = 4;  // keys per thread: their gathers are independent and overlap
     const int bh = blockIdx.y;
     const int b = bh / H, h = bh % H;
     const int idx = blockIdx.x * 256 + threadIdx.x;
-    const int j = idx / CPR, col = idx % CPR;
-    if (j >= N) return;
-    const uint8_t* code = codes + b * c_sb + h * c_sh + (int64_t)j * M;
-    float acc[8];
+    const int j0 = (idx / CPR) * KPT, col = idx % CPR;
+    if (j0 >= N) return;
+    const uint8_t* code = codes + b * c_sb + h * c_sh;
+    const uint16_t* cbh = cb + h * cb_sh + col * 8;
+    float acc[KPT][8];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+    for (int k = 0; k < KPT; ++k)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[k][e] = 0.f;
     for (int m = 0; m < M; ++m) {
-        const u32x4_t w = *reinterpret_cast<const u32x4_t*>(cb + h * cb_sh + m * cb_sm + (int64_t)code[m] * cb_sk +
-                                                            col * 8);
+        u32x4_t w[KPT];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            acc[2 * e] += Elem<Tag>::from_bits((uint16_t)(w[e] & 0xffffu));
-            acc[2 * e + 1] += Elem<Tag>::from_bits((uint16_t)(w[e] >> 16));
+        for (int k = 0; k < KPT; ++k) {
+            const int j = min(j0 + k, N - 1);
+            w[k] = *reinterpret_cast<const u32x4_t*>(cbh + m * cb_sm + (int64_t)code[(int64_t)j * M + m] * cb_sk);
         }
-    }
-    u32x4_t o;
 #pragma unroll
-    for (int e = 0; e < 4; ++e)
-        o[e] = (uint32_t)Elem<Tag>::to_bits(acc[2 * e]) | ((uint32_t)Elem<Tag>::to_bits(acc[2 * e + 1]) << 16);
-    *reinterpret_cast<u32x4_t*>(kc + ((int64_t)bh * N + j) * D + col * 8) = o;
+        for (int k = 0; k < KPT; ++k)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                acc[k][2 * e] += Elem<Tag>::from_bits((uint16_t)(w[k][e] & 0xffffu));
+                acc[k][2 * e + 1] += Elem<Tag>::from_bits((uint16_t)(w[k][e] >> 16));
+            }
+    }
+#pragma unroll
+    for (int k = 0; k < KPT; ++k) {
+        if (j0 + k >= N) break;
+        u32x4_t o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            o[e] = (uint32_t)Elem<Tag>::to_bits(acc[k][2 * e]) | ((uint32_t)Elem<Tag>::to_bits(acc[k][2 * e + 1]) << 16);
+        *reinterpret_cast<u32x4_t*>(kc + ((int64_t)bh * N + j0 + k) * D + col * 8) = o;
+    }
 }
 
 inline size_t prefill_workspace_bytes(int B, int H, int N, int D) {
@@ -443,7 +457,7 @@ int prefill(const void* q, const uint8_t* codes, const void* codebooks, const vo
         return VQA_ERR_MISALIGNED;
 
     uint16_t* kc = static_cast<uint16_t*>(workspace);
-    const int chunks = N * (D / 8);
+    const int chunks = ((N + 3) / 4) * (D / 8);  // one thread per 16-byte column of 4 consecutive keys
     const dim3 dq_grid((chunks + 255) / 256, B * H);
     if (D == 64)
         hipLaunchKernelGGL((dequant_kernel<Tag, 64>), dq_grid, dim3(256), 0, stream, codes,
