@@ -60,7 +60,8 @@ const char* vqa_strerror(int status);
  *   v         [B,H,N,D]  same type as q      strides[7..9]  = (b, h, n); each row 16-byte aligned
  *   out       [B,H,1,D]  same type as q      strides[10..11] = (b, h)
  *   lse       [B,H] float, base 2, nullable
- *   M in {1,2,4,8}, K <= 256, D in {64,128}.
+ *   M in {1,2,4,8}, K <= 256, D in {64,128}.  Codes must lie in [0, K); a code >= K is scored as codeword K - 1 (the
+ *   same clamp applies to vqa_prefill_*), it never reads outside the codebook.
  *   num_splits: KV splits per (b,h); <= 0 lets the library choose (vqa_decode_default_splits).
  *   workspace: >= vqa_decode_workspace_bytes(...) bytes of device memory, 256-byte aligned, owned by the caller.
  * ------------------------------------------------------------------------------------------------------------------ */

@@ -66,6 +66,51 @@ def test_decode_rejects_bad_arguments_before_any_launch(lib):
     assert call(q=16, cb=16, v=16, codes=4, ws_bytes=8) == -6  # VQA_ERR_WORKSPACE_TOO_SMALL
 
 
+def test_row_strides_beyond_the_32_bit_lane_offsets_are_rejected(lib):
+    """64 rows x stride x 2 bytes must fit the 32-bit per-lane offsets of the streaming / tile-copy loops; larger (or
+    negative) row strides are refused on the host, before any launch."""
+    big = 1 << 24
+    s = [0] * 12
+    s[9] = big  # v row stride of the coded decode
+    rc = lib.vqa_decode_bf16(16, 16, 16, 16, 16, None, 256, 1 << 30, 1, 1, 8, 128, 4, 256, _lib.strides_array(*s), 1.0,
+                             1, None)
+    assert rc == -7
+    s = [0] * 10
+    s[4] = big  # k row stride of the exact decode
+    rc = lib.vqa_decode_exact_bf16(16, 16, 16, 16, None, 256, 1 << 30, 1, 1, 8, 128, _lib.strides_array(*s), 1.0, 1,
+                                   None)
+    assert rc == -7
+    s = [128] * 18
+    s[8] = -128  # negative k1 row stride of the window kernel
+    rc = lib.vqa_local_attn_bf16(16, 16, 16, 16, 16, 16, None, 1, 1, 8, 128, _lib.strides_array(*s), 4, 0, 1.0, None)
+    assert rc == -7
+    s[8] = big
+    rc = lib.vqa_local_attn_bf16(16, 16, 16, 16, 16, 16, None, 1, 1, 8, 128, _lib.strides_array(*s), 4, 0, 1.0, None)
+    assert rc == -7
+    s = [128] * 23
+    s[10] = big  # v row stride of the prefill: refused before the reconstruction kernel is enqueued
+    rc = lib.vqa_prefill_bf16(16, 16, 16, 16, None, None, None, 16, None, 256, 1 << 30, 1, 1, 8, 128, 4, 256,
+                              _lib.strides_array(*s), 0, 0, 1, 1.0, None)
+    assert rc == -7
+
+
+def test_generation_after_a_512_entry_prefill_raises_instead_of_restarting():
+    """A cache that has recorded a prefill classifies the next seqlen_q == 1 call as a generation step whatever the
+    codebook size; with more than 256 entries (no uint8 codes) that step raises instead of attending over one token."""
+    import torch
+
+    from vqtree_amd.ops import attn_vq as A
+
+    H, C, D, N = 2, 512, 64, 700
+    cache = A.VectorQuantizedReRoPECache(256, torch.zeros(H, C, D, dtype=torch.bfloat16))
+    A._remember(cache, 0, torch.randint(0, C, (1, H, N)), torch.zeros(1, H, N, D, dtype=torch.bfloat16), N)
+    assert cache.get_seq_length() == N and cache.seen_tokens == N and cache.key_codes[0].dtype == torch.int16
+    assert int(cache.key_codes[0].max()) > 255
+    one = torch.zeros(1, H, 1, D, dtype=torch.bfloat16)
+    with pytest.raises(NotImplementedError):
+        A.dispatch_attn(one, one, one, torch.tensor([[N]]), cache)
+
+
 def test_ops_refuse_cpu_tensors():
     import torch
 

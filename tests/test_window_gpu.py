@@ -275,3 +275,39 @@ def test_vq_prefill_fp32_config1(B, H, N, D, M, K, causal):
     assert out.dtype == torch.float32
     assert (out.cpu() - want).abs().max() <= 1e-4
     assert (lse.cpu() - want_lse).abs().max() <= 1e-4
+
+
+# ------------------------------------------------------------------ reconstructed keys, bit for bit
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,K,D", [(1, 256, 128), (2, 256, 64), (4, 256, 128), (8, 256, 128), (4, 200, 64),
+                                   (16, 96, 128)])
+def test_reconstructed_keys_are_bit_exact(M, K, D, dtype):
+    """The code gathers of the prefill: the workspace of vqa_prefill_* holds K_hat = sum_m codebooks[h,m,code_m]
+    (fp32 sum in codebook order, rounded once).  Called through ctypes with a workspace of the test's own and compared
+    with the oracle's reconstruction by torch.equal."""
+    from vqtree_amd import _lib
+    from vqtree_amd.synthetic import prefill_case
+
+    _say(f"reconstructed keys M{M} K{K} D{D} {dtype}")
+    B, H, N = 2, 3, 333
+    case = prefill_case(B, H, N, D, M, 128, K=K, dtype=dtype, seed=40 + M)
+    lib = _lib.load()
+    sfx = {torch.bfloat16: "bf16", torch.float16: "f16"}[dtype]
+    ws_bytes = lib.vqa_prefill_workspace_bytes(B, H, N, D)
+    ws = torch.zeros(ws_bytes, dtype=torch.uint8, device="cuda")
+    out = torch.empty_like(case.q)
+    s3 = lambda t: (t.stride(0), t.stride(1), t.stride(2))
+    cb = case.codebooks
+    strides = _lib.strides_array(*s3(case.q), case.codes.stride(0), case.codes.stride(1), cb.stride(0), cb.stride(1),
+                                 cb.stride(2), *s3(case.v), *s3(case.k_exact), 0, 0, 0, 0, 0, 0, *s3(out))
+    rc = getattr(lib, "vqa_prefill_" + sfx)(case.q.data_ptr(), case.codes.data_ptr(), cb.data_ptr(), case.v.data_ptr(),
+                                            case.k_exact.data_ptr(), None, None, out.data_ptr(), None, ws.data_ptr(),
+                                            ws_bytes, B, H, N, D, M, K, strides, 128, 0, 1, case.softmax_scale,
+                                            _lib.current_stream(case.q.device))
+    _lib.check(rc)
+    torch.cuda.synchronize()
+    k_hat = ws[: B * H * N * D * 2].view(dtype).view(B, H, N, D).cpu()
+    want = oracle.reconstruct_keys(case.codes, cb).to(dtype)
+    assert torch.equal(k_hat, want)
+    want_out, _ = oracle.attn_vq_prefill(case.q, case.codes, cb, case.v, k_exact=case.k_exact, window_size=128)
+    assert_close_16(out, want_out, "prefill around the reconstruction")

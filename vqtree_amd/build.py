@@ -29,28 +29,32 @@ def sources():
     return sorted(glob.glob(os.path.join(CSRC_DIR, "*.hip")))
 
 
+def _compile(cmd):
+    # communicate() drains the compiler's output while it runs, so a long warning log cannot block the child
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    return proc.returncode, proc.stdout
+
+
 def build(verbose: bool = True, jobs: int = 8) -> str:
     """Compile every csrc/*.hip into objects (in parallel) and link the shared library.  Always recompiles."""
+    from concurrent.futures import ThreadPoolExecutor
+
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     obj_dir = os.path.join(PKG_DIR, "build")
     os.makedirs(obj_dir, exist_ok=True)
     flags = [f for f in HIPCC_FLAGS if f != "-shared"]
-    procs = []
-    objs = []
-    for src in sources():
-        obj = os.path.join(obj_dir, os.path.basename(src) + ".o")
-        objs.append(obj)
-        cmd = [hipcc, *flags, "-c", src, "-o", obj]
-        if verbose:
+    srcs = sources()
+    objs = [os.path.join(obj_dir, os.path.basename(src) + ".o") for src in srcs]
+    cmds = [[hipcc, *flags, "-c", src, "-o", obj] for src, obj in zip(srcs, objs)]
+    if verbose:
+        for cmd in cmds:
             print(" ".join(cmd), flush=True)
-        procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
-        while sum(p.poll() is None for _, p in procs) >= jobs:
-            procs[0][1].wait()
+    with ThreadPoolExecutor(max_workers=max(1, jobs)) as pool:
+        results = list(pool.map(_compile, cmds))
     failed = False
-    for src, p in procs:
-        out, _ = p.communicate()
+    for src, (rc, out) in zip(srcs, results):
         lines = [l for l in out.splitlines() if "is not a recognized feature for this target" not in l]
-        if p.returncode != 0:
+        if rc != 0:
             failed = True
             print(f"FAILED: {src}\n" + "\n".join(lines), file=sys.stderr)
         elif verbose and lines:

@@ -126,6 +126,10 @@ __device__ __forceinline__ void store_stream16(void* p, uint4 v) {
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+// Row strides (in elements of a 16-bit type) for which 64 consecutive rows still fit the 32-bit per-lane byte offsets
+// of the streaming and tile-copy loops; anything else is rejected on the host before a launch.
+inline bool row_stride_ok(int64_t sn) { return sn >= 0 && sn < (int64_t(1) << 24); }
+
 inline int launch_status() { return hipGetLastError() == hipSuccess ? VQA_OK : VQA_ERR_LAUNCH_FAILED; }
 
 }  // namespace vqa

@@ -82,7 +82,7 @@ __global__ __launch_bounds__(kThreads, 2) void count_kernel(CountParams p) {
     int64_t rows[TileCopy<D, true>::kInstr];
     float cnt_f = 0.f;
     auto fetch_meta = [&](int c0) {
-        v_copy.fetch_rows(rows, vi, c0, p.C);
+        v_copy.fetch_rows(rows, vi, c0, p.C, p.N);  // v_vq has N + 1 rows
         cnt_f = (tid < kBN && c0 + tid < p.C) ? Elem<Tag>::from_bits(cnt[c0 + tid]) : 0.f;  // 0: masked
     };
     auto request = [&](int c0, int buf) {  // uses the metadata fetched for c0
@@ -184,6 +184,7 @@ int vqcount(const void* q2, const void* k_vq, const void* k_vq_cnt, const void* 
     if (merge_into && !lse) return VQA_ERR_NULL_POINTER;
     if (B <= 0 || H <= 0 || N <= 0 || C <= 0) return VQA_ERR_BAD_SHAPE;
     if (window < 0 || !(sm_scale > 0.f) || (int64_t)B * H > 65535) return VQA_ERR_BAD_ARGUMENT;
+    if (!row_stride_ok(strides[2]) || !row_stride_ok(strides[4]) || !row_stride_ok(strides[10])) return VQA_ERR_BAD_ARGUMENT;
     CountParams p;
     p.q = View{static_cast<const uint16_t*>(q2), strides[0], strides[1], strides[2]};
     p.cb = static_cast<const uint16_t*>(k_vq);

@@ -37,8 +37,10 @@ __global__ __launch_bounds__(kThreads) void lut_kernel(const uint16_t* __restric
     typedef typename Elem<Tag>::vec8 vec8;
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int tile = blockIdx.x * kWaves + wave;  // 16-codeword tile inside this codebook
-    if (tile * 16 >= K) return;
+    // 16-codeword tile inside this codebook; all kLutStride entries are written, those past K repeat codeword K - 1,
+    // so a code >= K scores (deterministically) as K - 1
+    const int tile = blockIdx.x * kWaves + wave;
+    if (tile * 16 >= kLutStride) return;
     const int hm = blockIdx.y;
     const int h = hm / M, m = hm % M;
     const int r = lane & 15;   // A row (codeword) / B column (batch row)
@@ -62,8 +64,7 @@ __global__ __launch_bounds__(kThreads) void lut_kernel(const uint16_t* __restric
         if (bb < B) {
             float* dst = lut + ((int64_t)(bb * H + h) * M + m) * kLutStride + tile * 16 + kq * 4;
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-                if (tile * 16 + kq * 4 + i < K) dst[i] = acc[i] * scale_log2e;
+            for (int i = 0; i < 4; ++i) dst[i] = acc[i] * scale_log2e;
         }
     }
 }
@@ -538,7 +539,7 @@ int run_d(const void* q, const uint8_t* codes, const void* codebooks, const void
     const uint16_t* cb16 = static_cast<const uint16_t*>(codebooks);
     const uint16_t* v16 = static_cast<const uint16_t*>(v);
 
-    const int tiles = (K + 15) / 16;
+    const int tiles = kLutStride / 16;
     hipLaunchKernelGGL((lut_kernel<Tag, D>), dim3((tiles + kWaves - 1) / kWaves, H * M), dim3(kThreads), 0, stream,
                        q16, cb16, lut, B, H, M, K, st, sm_scale * kLog2e);
     int rc = launch_status();
@@ -579,6 +580,7 @@ int run(const void* q, const uint8_t* codes, const void* codebooks, const void* 
         return VQA_ERR_MISALIGNED;
     if ((st.q_b | st.q_h | st.cb_h | st.cb_m | st.cb_k | st.v_b | st.v_h | st.v_n) & 7) return VQA_ERR_MISALIGNED;
     if (((uintptr_t)codes | (uintptr_t)st.c_b | (uintptr_t)st.c_h) & (uintptr_t)(M - 1)) return VQA_ERR_MISALIGNED;
+    if (!row_stride_ok(st.v_n)) return VQA_ERR_BAD_ARGUMENT;
     int S = num_splits > 0 ? num_splits : default_splits(B, H, N);
     if (S > 65535 || (int64_t)B * H > 65535) return VQA_ERR_BAD_ARGUMENT;
     if (workspace_bytes < plan(B, H, D, M, S).total) return VQA_ERR_WORKSPACE_TOO_SMALL;
@@ -605,6 +607,7 @@ int run_exact(const void* q, const void* k, const void* v, void* out, float* lse
     st.o_b = strides[8], st.o_h = strides[9];
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || ((uintptr_t)workspace & 255u)) return VQA_ERR_MISALIGNED;
     if ((es.q_b | es.q_h | es.k_b | es.k_h | es.k_n | es.v_b | es.v_h | es.v_n) & 7) return VQA_ERR_MISALIGNED;
+    if (!row_stride_ok(es.k_n) || !row_stride_ok(es.v_n)) return VQA_ERR_BAD_ARGUMENT;
     const int S = num_splits > 0 ? num_splits : default_splits(B, H, N);
     if (S > 65535 || (int64_t)B * H > 65535) return VQA_ERR_BAD_ARGUMENT;
     const Workspace ws = plan(B, H, D, 0, S);
@@ -663,7 +666,7 @@ int run_windowed_d(const uint16_t* q_far, const uint16_t* q_win, const uint8_t* 
     int rc = VQA_OK;
     const int far = N - W;
     if (far > 0) {
-        const int tiles = (K + 15) / 16;
+        const int tiles = kLutStride / 16;
         hipLaunchKernelGGL((lut_kernel<Tag, D>), dim3((tiles + kWaves - 1) / kWaves, H * M), dim3(kThreads), 0, stream,
                            q_far, cb, lut, B, H, M, K, st, sm_scale * kLog2e);
         if ((rc = launch_status()) != VQA_OK) return rc;
@@ -713,7 +716,7 @@ int run_windowed(const void* q_far, const void* q_win, const uint8_t* codes, con
         return VQA_ERR_MISALIGNED;
     if (codes && (((uintptr_t)codes | (uintptr_t)st.c_b | (uintptr_t)st.c_h) & (uintptr_t)(M - 1)))
         return VQA_ERR_MISALIGNED;
-    if ((int64_t)B * H > 65535) return VQA_ERR_BAD_ARGUMENT;
+    if ((int64_t)B * H > 65535 || !row_stride_ok(st.v_n) || !row_stride_ok(es.k_n)) return VQA_ERR_BAD_ARGUMENT;
     int s_far, s_win;
     windowed_splits(B, H, N, W, s_far, s_win);
     if (workspace_bytes < plan(B, H, D, M, s_far + s_win).total) return VQA_ERR_WORKSPACE_TOO_SMALL;

@@ -204,6 +204,7 @@ int encode(const void* x, const void* codebooks, uint8_t* codes, int64_t* ids, i
     p.i_sb = strides[9], p.i_sh = strides[10], p.i_sn = strides[11];
     p.H = H, p.N = N, p.M = M, p.K = K;
     p.mode = mode, p.round_scores = round_scores;
+    if (!row_stride_ok(p.cb_sk)) return VQA_ERR_BAD_ARGUMENT;
     if (!aligned16(x) || !aligned16(codebooks) || ((p.x_sb | p.x_sh | p.x_sn | p.cb_sh | p.cb_sm | p.cb_sk) & 7))
         return VQA_ERR_MISALIGNED;
     const dim3 grid((N + kKeysPerBlock - 1) / kKeysPerBlock, B * H);

@@ -152,10 +152,14 @@ struct TileCopy {
     }
     // same with the global rows taken from an index list, in two steps so that the indices can be fetched a tile
     // ahead of the copy that uses them: rows[i] = row_index[n0 + row(i)] (clamped), then one copy per index
-    __device__ __forceinline__ void fetch_rows(int64_t (&rows)[kInstr], const int64_t* row_index, int n0,
-                                               int n_rows) const {
+    // (index values are clamped to [0, max_index], so a corrupt list cannot send the copy outside the matrix)
+    __device__ __forceinline__ void fetch_rows(int64_t (&rows)[kInstr], const int64_t* row_index, int n0, int n_rows,
+                                               int64_t max_index) const {
 #pragma unroll
-        for (int i = 0; i < kInstr; ++i) rows[i] = row_index[min(n0 + row(i), n_rows - 1)];
+        for (int i = 0; i < kInstr; ++i) {
+            const int64_t r = row_index[min(n0 + row(i), n_rows - 1)];
+            rows[i] = r < 0 ? 0 : (r > max_index ? max_index : r);
+        }
     }
     __device__ __forceinline__ void load_rows(const char* lds_tile, const uint16_t* base, int64_t sn,
                                               const int64_t (&rows)[kInstr]) const {

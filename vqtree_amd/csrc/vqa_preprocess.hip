@@ -214,12 +214,19 @@ int preprocess(const int64_t* ids, const void* v, int64_t* cnt, void* cnt_elem, 
     p.start = reinterpret_cast<int32_t*>(ws);
     ws += align256(bh * C * 4);
     p.order = reinterpret_cast<int32_t*>(ws);
+    int rc;
     hipLaunchKernelGGL(hist_kernel, dim3(p.NB, B * H), dim3(kBlock), C * sizeof(int), stream, p);
+    if ((rc = launch_status()) != VQA_OK) return rc;
     hipLaunchKernelGGL(cumulate_kernel, dim3((C + 255) / 256, B * H), dim3(256), 0, stream, p);
+    if ((rc = launch_status()) != VQA_OK) return rc;
     hipLaunchKernelGGL(start_kernel, dim3(B * H), dim3(256), 0, stream, p);
-    if (N / kBlock > 0)
+    if ((rc = launch_status()) != VQA_OK) return rc;
+    if (N / kBlock > 0) {
         hipLaunchKernelGGL((emit_kernel<Tag>), dim3((C + 255) / 256, N / kBlock, B * H), dim3(256), 0, stream, p);
+        if ((rc = launch_status()) != VQA_OK) return rc;
+    }
     hipLaunchKernelGGL(scatter_kernel, dim3(p.NB, B * H), dim3(kBlock), 0, stream, p);
+    if ((rc = launch_status()) != VQA_OK) return rc;
     hipLaunchKernelGGL((segment_sum_kernel<Tag>), dim3((C + 3) / 4, B * H), dim3(256), 0, stream, p);
     return launch_status();
 }

@@ -333,15 +333,26 @@ inline bool view_ok(const View& v) {
     return v.p != nullptr && aligned16(v.p) && ((v.sb | v.sh | v.sn) & 7) == 0;
 }
 
-template <typename Tag>
-int run(Params p, int B, int D, int mode, hipStream_t stream) {
+// every host-side check of a launch; nothing is enqueued before it passes
+inline int validate(const Params& p, int B, int D) {
     if (B <= 0 || p.H <= 0 || p.N <= 0) return VQA_ERR_BAD_SHAPE;
     if ((int64_t)B * p.H > 65535) return VQA_ERR_BAD_ARGUMENT;
     if (p.window < 0 || !(p.scale_log2e > 0.f)) return VQA_ERR_BAD_ARGUMENT;
+    if (D != 64 && D != 128) return VQA_ERR_UNSUPPORTED_HEAD_DIM;
     if (!view_ok(p.qa) || !view_ok(p.qb) || !view_ok(p.ka) || !view_ok(p.kb) || !view_ok(p.kc) || !view_ok(p.v))
         return (p.qa.p && p.qb.p && p.ka.p && p.kb.p && p.kc.p && p.v.p) ? VQA_ERR_MISALIGNED : VQA_ERR_NULL_POINTER;
+    if (!row_stride_ok(p.qa.sn) || !row_stride_ok(p.qb.sn) || !row_stride_ok(p.ka.sn) || !row_stride_ok(p.kb.sn) ||
+        !row_stride_ok(p.kc.sn) || !row_stride_ok(p.v.sn))
+        return VQA_ERR_BAD_ARGUMENT;
     if (!p.out) return VQA_ERR_NULL_POINTER;
     if (((uintptr_t)p.out & 7) || ((p.o_sb | p.o_sh | p.o_sn) & 3)) return VQA_ERR_MISALIGNED;
+    return VQA_OK;
+}
+
+template <typename Tag>
+int run(Params p, int B, int D, int mode, hipStream_t stream) {
+    const int rc = validate(p, B, D);
+    if (rc != VQA_OK) return rc;
     if (D == 64) return dispatch_mode<Tag, 64>(p, B, mode, stream);
     if (D == 128) return dispatch_mode<Tag, 128>(p, B, mode, stream);
     return VQA_ERR_UNSUPPORTED_HEAD_DIM;
@@ -385,8 +396,8 @@ int local_attn(const void* q1, const void* q2, const void* k1, const void* k2, c
 template <typename Tag, int D>
 __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict__ codes,
                                                       const uint16_t* __restrict__ cb, uint16_t* __restrict__ kc,
-                                                      int H, int N, int M, int64_t c_sb, int64_t c_sh, int64_t cb_sh,
-                                                      int64_t cb_sm, int64_t cb_sk) {
+                                                      int H, int N, int M, int K, int64_t c_sb, int64_t c_sh,
+                                                      int64_t cb_sh, int64_t cb_sm, int64_t cb_sk) {
     constexpr int CPR = D / 8;
     constexpr int KPT = 4;  // keys per thread: their gathers are independent and overlap
     const int bh = blockIdx.y;
@@ -406,7 +417,8 @@ __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict_
 #pragma unroll
         for (int k = 0; k < KPT; ++k) {
             const int j = min(j0 + k, N - 1);
-            w[k] = *reinterpret_cast<const u32x4_t*>(cbh + m * cb_sm + (int64_t)code[(int64_t)j * M + m] * cb_sk);
+            const int c = min((int)code[(int64_t)j * M + m], K - 1);  // a code >= K reads codeword K - 1
+            w[k] = *reinterpret_cast<const u32x4_t*>(cbh + m * cb_sm + (int64_t)c * cb_sk);
         }
 #pragma unroll
         for (int k = 0; k < KPT; ++k)
@@ -457,19 +469,6 @@ int prefill(const void* q, const uint8_t* codes, const void* codebooks, const vo
         return VQA_ERR_MISALIGNED;
 
     uint16_t* kc = static_cast<uint16_t*>(workspace);
-    const int chunks = ((N + 3) / 4) * (D / 8);  // one thread per 16-byte column of 4 consecutive keys
-    const dim3 dq_grid((chunks + 255) / 256, B * H);
-    if (D == 64)
-        hipLaunchKernelGGL((dequant_kernel<Tag, 64>), dq_grid, dim3(256), 0, stream, codes,
-                           static_cast<const uint16_t*>(codebooks), kc, H, N, M, s_c[0], s_c[1], s_cb[0], s_cb[1],
-                           s_cb[2]);
-    else
-        hipLaunchKernelGGL((dequant_kernel<Tag, 128>), dq_grid, dim3(256), 0, stream, codes,
-                           static_cast<const uint16_t*>(codebooks), kc, H, N, M, s_c[0], s_c[1], s_cb[0], s_cb[1],
-                           s_cb[2]);
-    int rc = launch_status();
-    if (rc != VQA_OK) return rc;
-
     Params p;
     p.qa = make_view(q, s_q);
     p.qb = q2 ? make_view(q2, s_q2) : p.qa;
@@ -485,6 +484,21 @@ int prefill(const void* q, const uint8_t* codes, const void* codebooks, const vo
     p.causal = causal;
     p.boundary = k_exact ? boundary_mode : kBoundaryAllFar;
     p.scale_log2e = sm_scale * kLog2e;
+    int rc = validate(p, B, D);
+    if (rc != VQA_OK) return rc;
+
+    const int chunks = ((N + 3) / 4) * (D / 8);  // one thread per 16-byte column of 4 consecutive keys
+    const dim3 dq_grid((chunks + 255) / 256, B * H);
+    if (D == 64)
+        hipLaunchKernelGGL((dequant_kernel<Tag, 64>), dq_grid, dim3(256), 0, stream, codes,
+                           static_cast<const uint16_t*>(codebooks), kc, H, N, M, K, s_c[0], s_c[1], s_cb[0], s_cb[1],
+                           s_cb[2]);
+    else
+        hipLaunchKernelGGL((dequant_kernel<Tag, 128>), dq_grid, dim3(256), 0, stream, codes,
+                           static_cast<const uint16_t*>(codebooks), kc, H, N, M, K, s_c[0], s_c[1], s_cb[0], s_cb[1],
+                           s_cb[2]);
+    rc = launch_status();
+    if (rc != VQA_OK) return rc;
     return run<Tag>(p, B, D, kVqPrefill, stream);
 }
 

@@ -412,19 +412,26 @@ def long_prefilling_per_key(query_states, key_states, value_states, position_ids
 
 
 def _remember(cache, layer_idx, ids, value_states, n_tokens):
+    """Record a prefill in the cache.  The values (and with them `get_seq_length`) are always recorded, so the next
+    seqlen_q == 1 call is recognised as a generation step whatever the codebook size; the key codes are kept as uint8
+    when the codebook has at most 256 entries (what `attn_vq_decode` streams), as int16 otherwise."""
     if layer_idx == 0:
         cache.seen_tokens += n_tokens
-    if len(cache.value_cache) <= layer_idx and cache.codebook.shape[1] <= 256:
-        cache.key_codes.append(ids.to(torch.uint8).unsqueeze(-1).contiguous())
+    if len(cache.value_cache) <= layer_idx:
+        code_dtype = torch.uint8 if cache.codebook.shape[1] <= 256 else torch.int16
+        cache.key_codes.append(ids.to(code_dtype).unsqueeze(-1).contiguous())
         cache.value_cache.append(value_states)
 
 
-def long_prefilling_slow_reference_impl(query_states, key_states, value_states, position_ids, cache, rope_base=10000.0):
-    """Per-query loops of ops/attn_vq.py:278-334, kept for checking the linear-time path (torch ops, any device)."""
+def long_prefilling_slow_reference_impl(query_states, key_states, value_states, position_ids, cache, layer_idx=0,
+                                        rope_base=10000.0):
+    """Per-query loops of ops/attn_vq.py:278-334, kept for checking the linear-time path (torch operators around the
+    HIP key encoder)."""
     B, H, N, D = query_states.shape
     W = cache.window_length
     q1, k1, q2 = rerope_operands(query_states, key_states, position_ids, W, rope_base)
-    k_hat, _, _ = multi_head_single_quantize(key_states, cache.codebook)
+    k_hat, ids, _ = multi_head_single_quantize(key_states, cache.codebook)
+    _remember(cache, layer_idx, ids, value_states, N)
     scale = 1.0 / math.sqrt(D)
     output = torch.zeros_like(query_states, memory_format=torch.contiguous_format)
     for b in range(B):
@@ -459,7 +466,7 @@ def dispatch_attn(query_states, key_states, value_states, position_ids, cache, l
                                                      layer_idx, rope_base)
         if cache.attention_mode == AttentionMode.SLOW_REFERNECE:
             return long_prefilling_slow_reference_impl(query_states, key_states, value_states, position_ids, cache,
-                                                       rope_base)
+                                                       layer_idx, rope_base)
         raise KeyError(f"Bad attention mode: {cache.attention_mode}")
     if is_prefilling:
         q1, k1, _ = rerope_operands(query_states, key_states, position_ids, cache.window_length, rope_base)
@@ -469,7 +476,10 @@ def dispatch_attn(query_states, key_states, value_states, position_ids, cache, l
         _remember(cache, layer_idx, ids, value_states, q_len)
         return out.contiguous().flatten(2)
     assert q_len == 1, "Only support prefilling or generation"
-    assert len(cache.key_codes) > layer_idx, "decode needs a codebook of at most 256 entries"
+    if cache.key_codes[layer_idx].dtype != torch.uint8:
+        raise NotImplementedError(
+            "generation after a prefill needs a codebook of at most 256 entries (uint8 key codes); this cache holds "
+            f"{cache.codebook.shape[1]}")
     # generation step: append the new key's code and value, then attend over all codes with the clamped query
     ids = quantize_ids(key_states, cache.codebook)
     cache.key_codes[layer_idx] = torch.cat([cache.key_codes[layer_idx], ids.to(torch.uint8).unsqueeze(-1)], dim=2)
