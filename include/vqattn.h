@@ -4,7 +4,8 @@
  * This is the boundary a host binds instead of the reference's Triton launches.  Every entry point
  *   - takes plain device pointers, sizes and element strides (no torch types),
  *   - enqueues its kernels on the given HIP stream and returns without synchronising,
- *   - allocates nothing and keeps no mutable global state (scratch comes in through `workspace`),
+ *   - allocates nothing and keeps no mutable global state (scratch comes in through `workspace`; the one exception,
+ *     vqa_decode_static_bf16, works in a fixed device array of the library and says so below),
  *   - returns VQA_OK (0) or a negative vqa_status; it never throws or aborts.
  * Tensors are addressed as base + sum(index_i * stride_i) in ELEMENTS of their own type; the innermost
  * (head_dim / codebook index M) stride must be 1.  Head dims of the attention entry points: 64 and 128 (the encoder,
@@ -37,7 +38,8 @@ typedef enum vqa_status {
     VQA_ERR_MISALIGNED = -5,
     VQA_ERR_WORKSPACE_TOO_SMALL = -6,
     VQA_ERR_BAD_ARGUMENT = -7,
-    VQA_ERR_LAUNCH_FAILED = -8
+    VQA_ERR_LAUNCH_FAILED = -8,
+    VQA_ERR_SCRATCH_LIMIT = -9
 } vqa_status;
 
 /* Library version (major * 10000 + minor * 100 + patch). */
@@ -223,6 +225,22 @@ int vqa_decode_devlen_f16(const void* q, const uint8_t* codes, const void* codeb
                           float* lse, void* workspace, size_t workspace_bytes, int B, int H, int N_max, int D, int M,
                           int K, const int64_t* strides, float sm_scale, int num_splits, const int32_t* n_keys_dev,
                           vqa_stream_t stream);
+
+/* vqa_decode_bf16 for callers that cannot allocate or hand over device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc): no workspace argument, the lookup table and the split states live
+ * in a fixed VQA_DECODE_STATIC_SCRATCH_BYTES array inside the library, one copy per GPU, held until the process ends.
+ * It has no counterpart in the reference.  Same arguments, kernels and results as vqa_decode_bf16 otherwise.
+ *   - a problem whose vqa_decode_workspace_bytes(...) exceeds VQA_DECODE_STATIC_SCRATCH_BYTES is refused with
+ *     VQA_ERR_SCRATCH_LIMIT before anything is enqueued;
+ *   - the first call on a device looks up the array's device address (hipGetSymbolAddress); make that call outside a
+ *     stream capture;
+ *   - every call on one GPU uses the same array: calls that may overlap on that GPU (different streams) race, calls
+ *     ordered on one stream do not.  Every byte a call reads from the array it has written itself before. */
+#define VQA_DECODE_STATIC_SCRATCH_BYTES (8u << 20)
+
+int vqa_decode_static_bf16(const void* q, const uint8_t* codes, const void* codebooks, const void* v, void* out,
+                           float* lse, int B, int H, int N, int D, int M, int K, const int64_t* strides, float sm_scale,
+                           int num_splits, vqa_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------------------------------
  * seqlen_q = 1 attention over exact keys: out[b,h] = softmax_j(sm_scale * <q[b,h], k[b,h,j]>) . v[b,h,j], no mask.

@@ -29,7 +29,7 @@ def test_version_and_error_strings(lib):
     assert lib.vqa_version() >= 100
     assert lib.vqa_strerror(0) == b"ok"
     seen = set()
-    for code in range(-8, 0):
+    for code in range(-9, 0):
         msg = lib.vqa_strerror(code)
         assert msg and msg != b"unknown vqa status" and msg not in seen
         seen.add(msg)
@@ -92,6 +92,12 @@ def test_row_strides_beyond_the_32_bit_lane_offsets_are_rejected(lib):
     rc = lib.vqa_prefill_bf16(16, 16, 16, 16, None, None, None, 16, None, 256, 1 << 30, 1, 1, 8, 128, 4, 256,
                               _lib.strides_array(*s), 0, 0, 1, 1.0, None)
     assert rc == -7
+
+
+def test_static_scratch_decode_refuses_oversized_problem_on_the_host(lib):
+    strides = _lib.strides_array(*([0] * 12))
+    rc = lib.vqa_decode_static_bf16(16, 16, 16, 16, 16, None, 16, 32, 1 << 20, 128, 4, 256, strides, 1.0, 64, None)
+    assert rc == -9 and b"static" in lib.vqa_strerror(rc)
 
 
 def test_generation_after_a_512_entry_prefill_raises_instead_of_restarting():

@@ -20,6 +20,7 @@ SIGNATURES = {
     "vqa_decode_workspace_bytes": (c_size_t, [c_int] * 7),
     "vqa_decode_bf16": (c_int, [_P] * 7 + [c_size_t] + [c_int] * 6 + [_STRIDES, c_float, c_int, _P]),
     "vqa_decode_f16": (c_int, [_P] * 7 + [c_size_t] + [c_int] * 6 + [_STRIDES, c_float, c_int, _P]),
+    "vqa_decode_static_bf16": (c_int, [_P] * 6 + [c_int] * 6 + [_STRIDES, c_float, c_int, _P]),
     "vqa_decode_devlen_bf16": (c_int, [_P] * 7 + [c_size_t] + [c_int] * 6 + [_STRIDES, c_float, c_int, _P, _P]),
     "vqa_decode_devlen_f16": (c_int, [_P] * 7 + [c_size_t] + [c_int] * 6 + [_STRIDES, c_float, c_int, _P, _P]),
     "vqa_decode_windowed_workspace_bytes": (c_size_t, [c_int] * 6),

@@ -16,6 +16,8 @@ const char* vqa_strerror(int status) {
         case VQA_ERR_WORKSPACE_TOO_SMALL: return "workspace is smaller than the *_workspace_bytes query reports";
         case VQA_ERR_BAD_ARGUMENT: return "argument out of range";
         case VQA_ERR_LAUNCH_FAILED: return "HIP kernel launch failed";
+        case VQA_ERR_SCRATCH_LIMIT:
+            return "problem needs more scratch than the static array of the allocation-free entry point holds";
         default: return "unknown vqa status";
     }
 }

@@ -7,6 +7,8 @@
 //                    writes one unnormalised partial state (o[D], m, l) per split
 //   3. merge_kernel  log-sum-exp merge of the split states, normalise, cast, optional lse
 // The main kernel is HBM-bound: per key it reads M code bytes and one D-element V row and nothing else.
+#include <mutex>
+
 #include "vqa_common.h"
 
 namespace vqa {
@@ -561,6 +563,36 @@ int run_d(const void* q, const uint8_t* codes, const void* codebooks, const void
     return launch_status();
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// Scratch of the allocation-free entry point (lookup table + split states): one copy per GPU, held until the process
+// ends.  Host code never passes `scratch` itself to a kernel -- the name is only a host-side handle -- but the device
+// address that hipGetSymbolAddress returns for the current device, looked up once per device.
+// ---------------------------------------------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[VQA_DECODE_STATIC_SCRATCH_BYTES];
+
+constexpr int kMaxDevices = 64;
+
+inline int static_scratch(void** out) {
+    static std::mutex mu;
+    static void* ptrs[kMaxDevices] = {};
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        (void)hipGetLastError();
+        return VQA_ERR_LAUNCH_FAILED;
+    }
+    std::lock_guard<std::mutex> lock(mu);
+    if (ptrs[dev] == nullptr) {
+        void* ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || ptr == nullptr) {
+            (void)hipGetLastError();
+            return VQA_ERR_LAUNCH_FAILED;
+        }
+        ptrs[dev] = ptr;
+    }
+    *out = ptrs[dev];
+    return VQA_OK;
+}
+
 template <typename Tag>
 int run(const void* q, const uint8_t* codes, const void* codebooks, const void* v, void* out, float* lse,
         void* workspace, size_t workspace_bytes, int B, int H, int N, int D, int M, int K, const int64_t* strides,
@@ -802,6 +834,20 @@ int vqa_decode_f16(const void* q, const uint8_t* codes, const void* codebooks, c
                    const int64_t* strides, float sm_scale, int num_splits, vqa_stream_t stream) {
     return vqa::decode::run<vqa::f16_tag>(q, codes, codebooks, v, out, lse, workspace, workspace_bytes, B, H, N, D, M,
                                           K, strides, sm_scale, num_splits, nullptr, stream);
+}
+
+int vqa_decode_static_bf16(const void* q, const uint8_t* codes, const void* codebooks, const void* v, void* out,
+                           float* lse, int B, int H, int N, int D, int M, int K, const int64_t* strides, float sm_scale,
+                           int num_splits, vqa_stream_t stream) {
+    // the size check comes first and needs no device: a problem beyond the static scratch is refused outright
+    if (B <= 0 || H <= 0 || N <= 0 || D <= 0 || M <= 0) return VQA_ERR_BAD_SHAPE;
+    const int S = num_splits > 0 ? num_splits : vqa::decode::default_splits(B, H, N);
+    if (vqa::decode::plan(B, H, D, M, S).total > (size_t)VQA_DECODE_STATIC_SCRATCH_BYTES) return VQA_ERR_SCRATCH_LIMIT;
+    void* ws = nullptr;
+    const int rc = vqa::decode::static_scratch(&ws);
+    if (rc != VQA_OK) return rc;
+    return vqa::decode::run<vqa::bf16_tag>(q, codes, codebooks, v, out, lse, ws, VQA_DECODE_STATIC_SCRATCH_BYTES, B, H,
+                                           N, D, M, K, strides, sm_scale, S, nullptr, stream);
 }
 
 int vqa_decode_devlen_bf16(const void* q, const uint8_t* codes, const void* codebooks, const void* v, void* out,
