@@ -154,6 +154,23 @@ int vqa_prefill_f16(const void* q, const uint8_t* codes, const void* codebooks, 
                     int B, int H, int N, int D, int M, int K, const int64_t* strides, int window, int boundary_mode,
                     int causal, float sm_scale, vqa_stream_t stream);
 
+/* The same prefill on the software-pipelined schedule (one wave per SIMD with 64 query rows, the exponentials of a key
+ * tile evaluated under the score MFMAs of the next one), for the reference's long-prefill configuration only: no second
+ * query / key pair, the block boundary rule, `window` a multiple of 128 (or k_exact == NULL: every key quantised).
+ * Anything else returns VQA_ERR_BAD_ARGUMENT.  Same strides array as vqa_prefill_* (the q2 / k2 slots are ignored), same
+ * workspace, same results within the 16-bit tolerance; on MI355X it runs level with vqa_prefill_* and is kept as the
+ * starting point for a schedule that overlaps softmax and matrix work inside one wave.  Counterpart in the reference: the
+ * two launches of ops/triton_fused_vq_attn.py:202-245. */
+int vqa_prefill_pipelined_bf16(const void* q, const uint8_t* codes, const void* codebooks, const void* v,
+                               const void* k_exact, void* out, float* lse, void* workspace, size_t workspace_bytes,
+                               int B, int H, int N, int D, int M, int K, const int64_t* strides, int window, int causal,
+                               float sm_scale, vqa_stream_t stream);
+
+int vqa_prefill_pipelined_f16(const void* q, const uint8_t* codes, const void* codebooks, const void* v,
+                              const void* k_exact, void* out, float* lse, void* workspace, size_t workspace_bytes,
+                              int B, int H, int N, int D, int M, int K, const int64_t* strides, int window, int causal,
+                              float sm_scale, vqa_stream_t stream);
+
 /* fp32 validation instantiation of the prefill: every visible key quantised (no exact window), plain fp32 FMA
  * arithmetic with the lookup-table formulation (LUT[i,m,c] = <q_i, codebooks[h,m,c]>, score = sum_m LUT[i,m,code_jm]);
  * checks the additive-code attention against a dense fp32 softmax to 1e-4.  q, v, out float [B,H,N,D]-addressable,

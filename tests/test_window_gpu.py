@@ -311,3 +311,36 @@ def test_reconstructed_keys_are_bit_exact(M, K, D, dtype):
     assert torch.equal(k_hat, want)
     want_out, _ = oracle.attn_vq_prefill(case.q, case.codes, cb, case.v, k_exact=case.k_exact, window_size=128)
     assert_close_16(out, want_out, "prefill around the reconstruction")
+
+
+# ------------------------------------------------------------------ software-pipelined schedule of the long prefill
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,H,N,D,M,W", [(1, 2, 1024, 128, 4, 256), (2, 2, 640, 64, 2, 128), (1, 2, 515, 128, 4, 128),
+                                          (1, 1, 300, 128, 4, 384), (1, 2, 777, 64, 8, 0), (2, 1, 1300, 128, 1, 1024),
+                                          (1, 3, 65, 128, 2, 128), (1, 1, 1, 128, 4, 128)])
+def test_vq_prefill_pipelined_schedule(B, H, N, D, M, W, dtype):
+    """vqa_prefill_pipelined_*: block boundary with a window that is a multiple of 128, or (W = 0 here) every key
+    quantised; against the oracle and against the default kernel."""
+    _say(f"vq prefill pipelined B{B} H{H} N{N} D{D} M{M} W{W} {dtype}")
+    q, k, v = (_randn(B, H, N, D, seed=90 + s, dtype=dtype) for s in range(3))
+    cb = _randn(H, M, 256, D, seed=95, std=0.35, dtype=dtype)
+    codes = _codes(B, H, N, M, seed=96)
+    kw = dict(k_exact=k, window_size=W) if W else {}
+    want, want_lse = oracle.attn_vq_prefill(q, codes, cb, v, **kw)
+    kw = {n: (t.cuda() if torch.is_tensor(t) else t) for n, t in kw.items()}
+    out, lse = attn_vq_prefill(q.cuda(), codes.cuda(), cb.cuda(), v.cuda(), return_lse=True, schedule="pipelined", **kw)
+    ref, _ = attn_vq_prefill(q.cuda(), codes.cuda(), cb.cuda(), v.cuda(), return_lse=True, **kw)
+    torch.cuda.synchronize()
+    assert_close_16(out, want, "pipelined vq prefill")
+    assert_close_lse(lse, want_lse, atol=1e-2)
+    assert (out.float() - ref.float()).abs().max() <= 2e-2
+
+
+def test_vq_prefill_pipelined_refuses_other_configurations():
+    from vqtree_amd._lib import VqaError
+
+    q, k, v = (_randn(1, 1, 256, 128, seed=s).cuda() for s in range(3))
+    cb = _randn(1, 2, 256, 128, seed=4, std=0.35).cuda()
+    codes = _codes(1, 1, 256, 2, seed=5).cuda()
+    with pytest.raises(VqaError):  # window not a multiple of 128
+        attn_vq_prefill(q, codes, cb, v, k_exact=k, window_size=100, schedule="pipelined")

@@ -48,11 +48,13 @@ struct Geom {
     static constexpr int kDBlocks = D / 32;                     // 32-row blocks of O^T
 
     // chunk-index XOR of a K tile row: 16 consecutive rows read the same logical chunk (ds_read_b128)
-    static __device__ __forceinline__ int swz_k(int row) { return (row / kRowsPerBankCycle) % kChunksPerRow; }
+    static __device__ __forceinline__ int swz_k(int row) {
+        return (int)(((unsigned)row / (unsigned)kRowsPerBankCycle) % (unsigned)kChunksPerRow);
+    }
     // chunk-index XOR of a V tile row: 8 consecutive rows x 4 consecutive chunks are read together
     // (ds_read_b64_tr_b16); even values only, so the two 8-byte halves of a chunk stay together
     static __device__ __forceinline__ int swz_v(int row) {
-        return 2 * ((row / kRowsPerBankCycle) % (kChunksPerRow / 2));
+        return (int)(2u * (((unsigned)row / (unsigned)kRowsPerBankCycle) % (unsigned)(kChunksPerRow / 2)));
     }
 };
 
@@ -114,8 +116,8 @@ struct TileCopy {
 
     __device__ __forceinline__ void init(int wave_, int lane) {
         wave = wave_;
-        lane_row = lane / Geom<D>::kChunksPerRow;
-        chunk = lane % Geom<D>::kChunksPerRow;
+        lane_row = (int)((unsigned)lane / (unsigned)Geom<D>::kChunksPerRow);
+        chunk = (int)((unsigned)lane % (unsigned)Geom<D>::kChunksPerRow);
 #pragma unroll
         for (int i = 0; i < kInstr; ++i) chunk_bytes[i] = (uint32_t)src_chunk(row(i)) * 16u;
     }

@@ -439,6 +439,13 @@ __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict_
     }
 }
 
+// the software-pipelined kernel for the long-prefill configuration (vqa_prefill_pipe.hip)
+bool prefill_pipe_applies(int window, int boundary_is_block, bool has_exact, bool has_second_pair);
+template <typename Tag>
+int prefill_pipe_run(const View& q, const View& ka, const View& kc, const View& v, uint16_t* out, int64_t o_sb,
+                     int64_t o_sh, int64_t o_sn, float* lse, int B, int H, int N, int D, int window, int causal,
+                     bool all_far, float scale_log2e, hipStream_t stream);
+
 inline size_t prefill_workspace_bytes(int B, int H, int N, int D) {
     return ((size_t)B * H * N * D * 2 + 255) / 256 * 256;
 }
@@ -448,8 +455,11 @@ template <typename Tag>
 int prefill(const void* q, const uint8_t* codes, const void* codebooks, const void* v, const void* k_exact,
             const void* q2, const void* k2, void* out, float* lse, void* workspace, size_t workspace_bytes, int B,
             int H, int N, int D, int M, int K, const int64_t* strides, int window, int boundary_mode, int causal,
-            float sm_scale, hipStream_t stream) {
+            float sm_scale, bool pipelined, hipStream_t stream) {
     if (!q || !codes || !codebooks || !v || !out || !workspace || !strides) return VQA_ERR_NULL_POINTER;
+    if (pipelined && !prefill_pipe_applies(window, boundary_mode == kBoundaryBlock, k_exact != nullptr,
+                                           k_exact && q2 && k2))
+        return VQA_ERR_BAD_ARGUMENT;
     if (B <= 0 || H <= 0 || N <= 0) return VQA_ERR_BAD_SHAPE;
     if (D != 64 && D != 128) return VQA_ERR_UNSUPPORTED_HEAD_DIM;
     if (M < 1 || M > 16 || K < 1 || K > 256) return VQA_ERR_UNSUPPORTED_CODEBOOK;
@@ -499,6 +509,9 @@ int prefill(const void* q, const uint8_t* codes, const void* codebooks, const vo
                            s_cb[2]);
     rc = launch_status();
     if (rc != VQA_OK) return rc;
+    if (pipelined)
+        return prefill_pipe_run<Tag>(p.qa, p.ka, p.kc, p.v, p.out, p.o_sb, p.o_sh, p.o_sn, p.lse, B, H, N, D, window,
+                                     causal, k_exact == nullptr, p.scale_log2e, stream);
     return run<Tag>(p, B, D, kVqPrefill, stream);
 }
 
@@ -548,7 +561,7 @@ int vqa_prefill_bf16(const void* q, const uint8_t* codes, const void* codebooks,
                      int causal, float sm_scale, vqa_stream_t stream) {
     return vqa::flash::prefill<vqa::bf16_tag>(q, codes, codebooks, v, k_exact, q2, k2, out, lse, workspace,
                                               workspace_bytes, B, H, N, D, M, K, strides, window, boundary_mode,
-                                              causal, sm_scale, stream);
+                                              causal, sm_scale, false, stream);
 }
 
 int vqa_prefill_f16(const void* q, const uint8_t* codes, const void* codebooks, const void* v, const void* k_exact,
@@ -557,7 +570,25 @@ int vqa_prefill_f16(const void* q, const uint8_t* codes, const void* codebooks, 
                     int causal, float sm_scale, vqa_stream_t stream) {
     return vqa::flash::prefill<vqa::f16_tag>(q, codes, codebooks, v, k_exact, q2, k2, out, lse, workspace,
                                              workspace_bytes, B, H, N, D, M, K, strides, window, boundary_mode, causal,
-                                             sm_scale, stream);
+                                             sm_scale, false, stream);
+}
+
+int vqa_prefill_pipelined_bf16(const void* q, const uint8_t* codes, const void* codebooks, const void* v,
+                               const void* k_exact, void* out, float* lse, void* workspace, size_t workspace_bytes,
+                               int B, int H, int N, int D, int M, int K, const int64_t* strides, int window, int causal,
+                               float sm_scale, vqa_stream_t stream) {
+    return vqa::flash::prefill<vqa::bf16_tag>(q, codes, codebooks, v, k_exact, nullptr, nullptr, out, lse, workspace,
+                                              workspace_bytes, B, H, N, D, M, K, strides, window,
+                                              vqa::flash::kBoundaryBlock, causal, sm_scale, true, stream);
+}
+
+int vqa_prefill_pipelined_f16(const void* q, const uint8_t* codes, const void* codebooks, const void* v,
+                              const void* k_exact, void* out, float* lse, void* workspace, size_t workspace_bytes,
+                              int B, int H, int N, int D, int M, int K, const int64_t* strides, int window, int causal,
+                              float sm_scale, vqa_stream_t stream) {
+    return vqa::flash::prefill<vqa::f16_tag>(q, codes, codebooks, v, k_exact, nullptr, nullptr, out, lse, workspace,
+                                             workspace_bytes, B, H, N, D, M, K, strides, window,
+                                             vqa::flash::kBoundaryBlock, causal, sm_scale, true, stream);
 }
 
 }  // extern "C"

@@ -142,7 +142,7 @@ def attn_vq_decode_windowed(q, k_codes, codebooks, v, k_window, *, softmax_scale
 
 
 def attn_vq_prefill(q, k_codes, codebooks, v, *, k_exact=None, window_size=0, causal=True, softmax_scale=None,
-                    return_lse=False, boundary_mode="block", q2=None, k2=None):
+                    return_lse=False, boundary_mode="block", q2=None, k2=None, schedule="default"):
     """Prefill attention (seqlen_q == seqlen_k) over additive-quantiser key codes, optionally with an exact window.
 
     q, v [B,H,N,D] bf16/f16; k_codes [B,H,N,M] uint8; codebooks [H,M,K,D].  With `k_exact` [B,H,N,D]: keys
@@ -151,6 +151,7 @@ def attn_vq_prefill(q, k_codes, codebooks, v, *, k_exact=None, window_size=0, ca
     with q2 if given else q.  boundary(i) = max(0, floor((i - W)/128)*128) for boundary_mode "block" (the rule of
     ops/attn_vq.py:311 and of the window kernel stages), max(0, i - W) for "exact".  One softmax over all visible
     keys: the window and far parts are merged inside the kernel.  Returns out [B,H,N,D] (and base-2 lse [B,H,N]).
+    `schedule="pipelined"` runs the software-pipelined kernel (block boundary, window a multiple of 128, no q2 / k2).
     """
     from ._common import BOUNDARY, bhn_strides, check_same_16bit, last_dim_contiguous, ptr
 
@@ -182,11 +183,19 @@ def attn_vq_prefill(q, k_codes, codebooks, v, *, k_exact=None, window_size=0, ca
         *(bhn_strides(k2) if k2 is not None else dummy),
         *bhn_strides(out),
     )
+    assert schedule in ("default", "pipelined")
     with torch.cuda.device(q.device):
-        rc = getattr(lib, "vqa_prefill_" + sfx)(
-            ptr(q), ptr(k_codes), ptr(codebooks), ptr(v), ptr(k_exact), ptr(q2), ptr(k2), ptr(out), ptr(lse),
-            ptr(workspace), ws_bytes, B, H, N, D, M, K, strides, int(window_size), BOUNDARY[boundary_mode],
-            1 if causal else 0, softmax_scale, _lib.current_stream(q.device))
+        if schedule == "pipelined":
+            assert q2 is None and k2 is None and boundary_mode == "block"
+            rc = getattr(lib, "vqa_prefill_pipelined_" + sfx)(
+                ptr(q), ptr(k_codes), ptr(codebooks), ptr(v), ptr(k_exact), ptr(out), ptr(lse), ptr(workspace),
+                ws_bytes, B, H, N, D, M, K, strides, int(window_size), 1 if causal else 0, softmax_scale,
+                _lib.current_stream(q.device))
+        else:
+            rc = getattr(lib, "vqa_prefill_" + sfx)(
+                ptr(q), ptr(k_codes), ptr(codebooks), ptr(v), ptr(k_exact), ptr(q2), ptr(k2), ptr(out), ptr(lse),
+                ptr(workspace), ws_bytes, B, H, N, D, M, K, strides, int(window_size), BOUNDARY[boundary_mode],
+                1 if causal else 0, softmax_scale, _lib.current_stream(q.device))
     _lib.check(rc)
     return (out, lse) if return_lse else out
 
