@@ -18,9 +18,14 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
-# HBM bytes one launch of the streaming kernel moves, from rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by a known copy
-# (profiles/decode_main_kernel_c2_b16_h32_n32768.md); valid for the default workload only
-DECODE_MAIN_KERNEL_TRAFFIC_BYTES = 4_380_977_000
+# HBM bytes one launch of the streaming kernel moves at the default workload: a counter measurement (rocprofv3
+# FETCH_SIZE / WRITE_SIZE scaled by a 1 GiB copy in the same run), not something this script can observe; the figure
+# and the file that documents the run that produced it travel together
+DECODE_MAIN_KERNEL_TRAFFIC = {
+    "bytes": 4_380_977_000,
+    "source": "profiles/decode_main_kernel_c2_b16_h32_n32768.md (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE; "
+              "not measured by this run)",
+}
 
 
 def cpu_baseline(case, units=256, repeats=5):
@@ -66,6 +71,19 @@ def cpu_baseline(case, units=256, repeats=5):
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 
 
+def _cpu_time(fn, repeats=3):
+    import torch
+
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    times = []
+    for _ in range(repeats):
+        t0 = time.perf_counter()
+        fn()
+        times.append(time.perf_counter() - t0)
+    return sorted(times)[len(times) // 2], cores
+
+
 def _time_events(fn, steps, warmup):
     import torch
 
@@ -83,7 +101,7 @@ def _time_events(fn, steps, warmup):
     return ms[len(ms) // 2]
 
 
-def prefill_extra(dev, steps=20, warmup=5):
+def prefill_extra(dev, steps=20, warmup=5, cpu=True):
     """Second half of the metric: causal VQ-attention prefill at 8k with a 1024-key exact window (not part of the
     timed decode region).  Reported as algorithmic TFLOP/s and as a fraction of the bf16 MFMA peak."""
     import torch
@@ -109,12 +127,26 @@ def prefill_extra(dev, steps=20, warmup=5):
                      "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
                      "duration_covers": "whole call: key reconstruction kernel + fused window/far attention kernel"},
     }
+    if cpu:
+        # the oracle on one of the H independent heads (same inputs), rate extrapolated over heads
+        import oracle
+
+        h = 0
+        args = [x[:, h:h + 1].cpu() for x in (case.q, case.codes)] + [case.codebooks[h:h + 1].cpu(), case.v[:, h:h + 1].cpu()]
+        k_ex = case.k_exact[:, h:h + 1].cpu()
+        t, cores = _cpu_time(lambda: oracle.attn_vq_prefill(*args, k_exact=k_ex, window_size=case.window,
+                                                            softmax_scale=case.softmax_scale), repeats=3)
+        out["cpu_baseline"] = {
+            "value": round(flops / (B * H) / t / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "sample": f"1 of {B * H} (batch, head) units of the same workload (heads are independent, rate "
+                      f"extrapolated), fp32 PyTorch oracle, median of 3 runs, {t * 1e3:.0f} ms",
+        }
     del case
     torch.cuda.empty_cache()
     return out
 
 
-def local_rerope_extra(dev, steps=10, warmup=3):
+def local_rerope_extra(dev, steps=10, warmup=3, cpu=True):
     """Sliding-window ReRoPE attention at 16k (batch 2, 32 heads, window 512), the exact-window building block of the
     prefill path: useful FLOPs = 4 * D * visible pairs (keys j <= i with j >= floor(i/128)*128 - window)."""
     import torch
@@ -141,7 +173,21 @@ def local_rerope_extra(dev, steps=10, warmup=3):
         "useful_gflop": round(flops / 1e9, 1),
         "tflops": round(tf, 1),
         "mfma_frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
+        "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4), "duration_covers": "the one window kernel"},
     }
+    if cpu:
+        import oracle
+
+        b, h = 0, 0
+        args = [x[b:b + 1, :, h:h + 1].transpose(1, 2).cpu() for x in (q1, k1, v)]
+        q2c, kc = (x[b:b + 1, :, h:h + 1].transpose(1, 2).cpu() for x in (q2, k))
+        t, cores = _cpu_time(lambda: oracle.local_attn(*args, W, "rerope", None, q2=q2c, k2=kc), repeats=3)
+        out["cpu_baseline"] = {
+            "value": round(flops / (B * H) / t / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "sample": f"1 of {B * H} (batch, head) units of the same workload (units are independent, rate "
+                      f"extrapolated), fp32 PyTorch oracle with dense masks, median of 3 runs, {t * 1e3:.0f} ms",
+        }
     del q, k, v, q1, k1, q2
     torch.cuda.empty_cache()
     return out
@@ -154,6 +200,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-prefill", action="store_true", help="skip the (untimed-region) prefill measurement")
+    ap.add_argument("--no-c5", action="store_true", help="skip the (untimed-region) 32-layer decode harness")
+    ap.add_argument("--c5-steps", type=int, default=16)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="before the timed region, run one plain 1 GiB device copy (reference dispatch of known "
                          "size for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE counters)")
@@ -232,7 +280,8 @@ def main():
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
-            "traffic": DECODE_MAIN_KERNEL_TRAFFIC_BYTES,
+            "traffic": DECODE_MAIN_KERNEL_TRAFFIC["bytes"],
+            "traffic_source": DECODE_MAIN_KERNEL_TRAFFIC["source"],
             "kernel": "vqa::decode::main_kernel<bf16,128,4>",
             "duration_us": round(kern_ms * 1e3, 1),
             "duration_covers": "HIP events around the whole call (lookup-table + streaming + merge kernels); the "
@@ -241,11 +290,21 @@ def main():
     }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(case)
+    del case
+    torch.cuda.empty_cache()
     if not args.no_prefill:
-        del case
-        torch.cuda.empty_cache()
-        result["prefill"] = prefill_extra(dev)
-        result["local_rerope"] = local_rerope_extra(dev)
+        result["prefill"] = prefill_extra(dev, cpu=not args.no_cpu_baseline)
+        result["local_rerope"] = local_rerope_extra(dev, cpu=not args.no_cpu_baseline)
+    if not args.no_c5:
+        # configuration 5: 32-layer Llama-2-7B-shaped greedy decode over per-layer VQ key caches at 65536 context
+        from vqtree_amd import decode_harness
+
+        c5 = decode_harness.run(steps=args.c5_steps, warmup=2)
+        c5["roofline"] = {"bound": "hbm", "achieved": c5["attention_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                          "frac": c5["attention_hbm_frac"],
+                          "duration_covers": "HIP events around the attention calls of all 32 layers (clamped query, "
+                                             "lookup table, streaming kernel, merge), per decode step"}
+        result["c5"] = c5
     print(json.dumps(result))
 
 

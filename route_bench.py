@@ -1,17 +1,23 @@
 """Timing of the reference-shaped long-prefill route (single codebook per head, count-weighted far context) and of its
 stages, next to the fused per-key formulation, at the prefill benchmark shape.
 
-    python -m vqtree_amd.route_bench [--heads 32 --tokens 8192 --window 1024 --codes 512]
+    python route_bench.py [--heads 32 --tokens 8192 --window 1024 --codes 512]
 
 Prints one JSON object; times are medians of HIP-event intervals in microseconds."""
 import argparse
 import json
+import os
+import sys
 
 import torch
 
-from .ops import attn_vq as A
-from .ops import mini_vq as Q
-from .ops.triton_fused_vq_attn import vq_attn_forward
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+from vqtree_amd.ops import attn_vq as A  # noqa: E402
+from vqtree_amd.ops import mini_vq as Q  # noqa: E402
+from vqtree_amd.ops.triton_fused_vq_attn import vq_attn_forward  # noqa: E402
 
 
 def _time(fn, steps=10, warmup=3):
@@ -50,6 +56,9 @@ def run(batch=1, heads=32, tokens=8192, head_dim=128, window=1024, codes=512, de
     cb256 = cb[:, :256].contiguous()
     ids256 = Q.quantize_ids(k, cb256).to(torch.uint8).unsqueeze(-1)
     out["fused_per_key_256_codewords_us"] = _time(
+        lambda: A.attn_vq_prefill(q1, ids256, cb256.unsqueeze(1), v, k_exact=k1, window_size=W, q2=q2, k2=k,
+                                  schedule="per_key"))
+    out["attn_vq_prefill_default_256_codewords_us"] = _time(  # M = 1: dispatched to the codeword-space route
         lambda: A.attn_vq_prefill(q1, ids256, cb256.unsqueeze(1), v, k_exact=k1, window_size=W, q2=q2, k2=k))
     return out
 

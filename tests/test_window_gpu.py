@@ -344,3 +344,25 @@ def test_vq_prefill_pipelined_refuses_other_configurations():
     codes = _codes(1, 1, 256, 2, seed=5).cuda()
     with pytest.raises(VqaError):  # window not a multiple of 128
         attn_vq_prefill(q, codes, cb, v, k_exact=k, window_size=100, schedule="pipelined")
+
+
+@pytest.mark.parametrize("with_rerope", [False, True])
+@pytest.mark.parametrize("B,H,N,D,K,W", [(1, 2, 1024, 128, 256, 256), (2, 2, 900, 64, 128, 128), (1, 1, 700, 128, 200, 384)])
+def test_single_codebook_prefill_takes_the_codeword_route(B, H, N, D, K, W, with_rerope):
+    """M = 1 with the block boundary: `attn_vq_prefill` runs the window kernel + count-weighted codeword kernel (far
+    context in O(N*K)); same oracle, and the per-key kernel forced on the same inputs agrees."""
+    _say(f"single-codebook prefill B{B} H{H} N{N} D{D} K{K} W{W} rerope={with_rerope}")
+    q, k, v, q2, k2 = (_randn(B, H, N, D, seed=110 + s) for s in range(5))
+    cb = _randn(H, 1, K, D, seed=115, std=0.5)
+    codes = _codes(B, H, N, 1, K, seed=116)
+    kw = dict(k_exact=k, window_size=W)
+    if with_rerope:
+        kw.update(q2=q2, k2=k2)
+    want, want_lse = oracle.attn_vq_prefill(q, codes, cb, v, **kw)
+    kw = {n: (t.cuda() if torch.is_tensor(t) else t) for n, t in kw.items()}
+    out, lse = attn_vq_prefill(q.cuda(), codes.cuda(), cb.cuda(), v.cuda(), return_lse=True, **kw)
+    per_key = attn_vq_prefill(q.cuda(), codes.cuda(), cb.cuda(), v.cuda(), schedule="per_key", **kw)
+    torch.cuda.synchronize()
+    assert_close_16(out, want, "codeword-route prefill")
+    assert_close_lse(lse, want_lse, atol=1e-2)
+    assert_close_16(per_key, want, "per-key prefill, M = 1")

@@ -19,7 +19,7 @@ import time
 
 import torch
 
-from .ops.attn_vq import attn_vq_decode, attn_vq_decode_windowed, rope_tables, rotate_half
+from .ops.attn_vq import apply_rope, attn_vq_decode, attn_vq_decode_windowed, rope_tables, rotate_half
 from .ops.mini_vq import RESIDUAL, encode_keys
 
 
@@ -85,7 +85,7 @@ class VQDecodeModel:
         """Attention of the new token (cache rows [0, n] are filled).  Coded keys are scored with the query at the
         clamped position window + 1, exact window keys with the query at its true position n."""
         scale = 1.0 / math.sqrt(self.D)
-        q_far = (q_raw * self.cos_w + rotate_half(q_raw) * self.sin_w).unsqueeze(2)  # [B,H,1,D]
+        q_far = apply_rope(q_raw.unsqueeze(2), self.cos, self.sin, self.window + 1)  # [B,H,1,D], one launch
         codes, values = layer["codes"][:, :, : n + 1], layer["values"][:, :, : n + 1]
         if not self.exact_window:
             return (attention or attn_vq_decode)(q_far, codes, layer["codebooks"], values, softmax_scale=scale)
@@ -158,7 +158,7 @@ class VQDecodeModel:
             h = self._rms(x)
             qkv = (h @ layer["wqkv"]).view(B, 3, H, D)
             q, k, v = qkv[:, 0], qkv[:, 1], qkv[:, 2]
-            q2 = (q * self.cos_w + rotate_half(q) * self.sin_w).unsqueeze(2)
+            q2 = apply_rope(q.unsqueeze(2), self.cos, self.sin, self.window + 1)
             layer["codes"].index_copy_(2, self.pos_dev, encode_residual(k.unsqueeze(2), layer["codebooks"]))
             layer["values"].index_copy_(2, self.pos_dev, v.unsqueeze(2))
             attn_vq_decode(q2, layer["codes"], layer["codebooks"], layer["values"], softmax_scale=1.0 / math.sqrt(D),

@@ -151,7 +151,9 @@ def attn_vq_prefill(q, k_codes, codebooks, v, *, k_exact=None, window_size=0, ca
     with q2 if given else q.  boundary(i) = max(0, floor((i - W)/128)*128) for boundary_mode "block" (the rule of
     ops/attn_vq.py:311 and of the window kernel stages), max(0, i - W) for "exact".  One softmax over all visible
     keys: the window and far parts are merged inside the kernel.  Returns out [B,H,N,D] (and base-2 lse [B,H,N]).
-    `schedule="pipelined"` runs the software-pipelined kernel (block boundary, window a multiple of 128, no q2 / k2).
+    `schedule`: "default" picks the kernel (one codebook with a block boundary: the codeword-space route of
+    `vq_attn_forward`; otherwise the per-key kernel), "per_key" forces the per-key kernel, "pipelined" runs its
+    software-pipelined variant (block boundary, window a multiple of 128, no q2 / k2).
     """
     from ._common import BOUNDARY, bhn_strides, check_same_16bit, last_dim_contiguous, ptr
 
@@ -165,6 +167,18 @@ def attn_vq_prefill(q, k_codes, codebooks, v, *, k_exact=None, window_size=0, ca
     assert causal or k_exact is None, "non-causal attention takes quantised keys only"
     if q.dtype == torch.float32:
         return _attn_vq_prefill_f32(q, k_codes, codebooks, v, k_exact, q2, k2, causal, softmax_scale, return_lse)
+    if (schedule == "default" and M == 1 and k_exact is not None and causal and boundary_mode == "block"
+            and (q2 is None) == (k2 is None) and window_size % BLOCK_SIZE == 0 and N > window_size + BLOCK_SIZE):
+        # One codebook: the far context is a softmax over the K codewords weighted by per-code key counts -- cost
+        # O(N * K) instead of O(N^2) -- which is the reference's own formulation (ops/triton_fused_vq_attn.py:22-70).
+        # The per-key kernel below only wins its place from M = 2 on (profiles/prefill_far_path_choice.md).
+        from .triton_fused_vq_attn import vq_attn_forward
+
+        ids = k_codes[..., 0].to(torch.int64)
+        cnt, v_vq, vi = segmented_preprocess(ids, v, K)
+        return vq_attn_forward(q, q if q2 is None else q2, k_exact, codebooks[:, 0], cnt,
+                               k_exact if (q2 is None or k2 is None) else k2, v, v_vq, vi, window_size,
+                               softmax_scale=softmax_scale, return_lse=return_lse)
     sfx = check_same_16bit(q, codebooks, v, k_exact, q2, k2)
     q, codebooks, v, k_exact, q2, k2 = last_dim_contiguous(q, codebooks, v, k_exact, q2, k2)
     if k_codes.stride(3) != 1 or k_codes.stride(2) != M:
@@ -183,7 +197,7 @@ def attn_vq_prefill(q, k_codes, codebooks, v, *, k_exact=None, window_size=0, ca
         *(bhn_strides(k2) if k2 is not None else dummy),
         *bhn_strides(out),
     )
-    assert schedule in ("default", "pipelined")
+    assert schedule in ("default", "per_key", "pipelined")
     with torch.cuda.device(q.device):
         if schedule == "pipelined":
             assert q2 is None and k2 is None and boundary_mode == "block"
@@ -415,7 +429,7 @@ def long_prefilling_per_key(query_states, key_states, value_states, position_ids
     q1, k1, q2 = rerope_operands(query_states, key_states, position_ids, cache.window_length, rope_base)
     out = attn_vq_prefill(q1, ids.to(torch.uint8).unsqueeze(-1), cache.codebook.unsqueeze(1), value_states,
                           k_exact=k1, window_size=cache.window_length, q2=q2, k2=key_states,
-                          softmax_scale=1 / math.sqrt(D))
+                          softmax_scale=1 / math.sqrt(D), schedule="per_key")
     _remember(cache, layer_idx, ids, value_states, N)
     return out.transpose(1, 2).contiguous().flatten(2)
 

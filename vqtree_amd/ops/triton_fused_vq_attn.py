@@ -55,10 +55,11 @@ def vq_count_forward(q2, k_vq, k_vq_cnt, v_vq, vi, window_size, softmax_scale=No
     return o2, l2
 
 
-def vq_attn_forward(q1, q2, k1, k_vq, k_vq_cnt, k3, v, v_vq, vi, window_size, softmax_scale=None):
+def vq_attn_forward(q1, q2, k1, k_vq, k_vq_cnt, k3, v, v_vq, vi, window_size, softmax_scale=None, return_lse=False):
     """q1/k1: rotary at true positions; q2: query at the clamped position; k_vq [H,C,D] codebook; k_vq_cnt / vi
     [B,H,N//128,C] running counts / prefix-sum row indices sampled per 128-key block; k3 raw keys; v_vq [B,H,N+1,D]
-    per-code prefix sums of V.  All attention tensors [B,H,N,D].  Returns [B,H,N,D].
+    per-code prefix sums of V.  All attention tensors [B,H,N,D].  Returns [B,H,N,D] (with `return_lse`, an extension,
+    also the merged base-2 log-sum-exp [B,H,N]).
 
     Unlike the reference (batch == 1 only, four layout copies around a separate merge launch) the two kernels work on
     the [B,H,N,D] tensors in place, the merge is the count kernel's epilogue, and any batch size is accepted.
@@ -69,4 +70,4 @@ def vq_attn_forward(q1, q2, k1, k_vq, k_vq_cnt, k3, v, v_vq, vi, window_size, so
     o1, l1 = local_attention_bhnd(q1, q2, k1, k3, v, window_size, LOCAL_REROPE, softmax_scale, True)
     # far context, merged into (o1, l1) by the count kernel's epilogue
     _count_call(q2, k_vq, k_vq_cnt, v_vq, vi, window_size, softmax_scale, o1, l1, merge=True)
-    return o1
+    return (o1, l1) if return_lse else o1
