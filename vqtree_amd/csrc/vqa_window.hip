@@ -191,15 +191,29 @@ __global__ __launch_bounds__(kThreads, 2) void window_kernel(Params p) {
     const int hi_key = rules.is_causal() ? min(p.N, m1 + 1) : p.N;
     const int u_hi = (hi_key + kBN - 1) / kBN;
     const int u_lo = max(0, rules.vis_lo(m0)) / kBN;
+    // Sliding-window modes: neighbouring query tiles share most of their key tiles, and the workgroups of an XCD that
+    // run at the same time are neighbours.  If each started at its own first key tile, a key tile would be read by
+    // its (window / 128 + 1) users several steps apart, with megabytes of other tiles in between -- more than the L2
+    // holds, so it would come from memory again for each of them.  Instead every workgroup walks its window in the
+    // same rotated order, key tile index modulo the number of tiles in a window: at any step all of them are on
+    // tiles of the same residue, so the users of one tile read it at about the same time.  (The online softmax does
+    // not care about the order.)  The walk is [u0, u_hi) followed by [u_lo, u0).
+    constexpr bool kRotate = (MODE == kLocalStrict || MODE == kLocalLoose || MODE == kLocalRerope);
+    int u0 = u_lo;
+    if (kRotate) {
+        const int period = (rules.W + kBM + kBN - 1) / kBN;
+        u0 = (u_lo + period - 1) / period * period;
+        if (u0 >= u_hi) u0 = u_lo;
+    }
 
     SoftmaxState<D> st;
     st.init();
 
     int buf = 0;  // buffer holding the tile about to be computed: K of its main pair, and V
     {
-        const int src = classify<MODE>(rules, m0, m1, u_lo * kBN).main;
-        k_copy.load(s_k[0], k_ptr(src), k_stride(src), u_lo * kBN, p.N);
-        v_copy.load(s_v[0], v_src, p.v.sn, u_lo * kBN, p.N);
+        const int src = classify<MODE>(rules, m0, m1, u0 * kBN).main;
+        k_copy.load(s_k[0], k_ptr(src), k_stride(src), u0 * kBN, p.N);
+        v_copy.load(s_v[0], v_src, p.v.sn, u0 * kBN, p.N);
     }
 
     // scores -> probabilities -> O update for the tile whose K / V sit in cur_k / cur_v
@@ -209,14 +223,16 @@ __global__ __launch_bounds__(kThreads, 2) void window_kernel(Params p) {
         pv_mma<Tag, D>(st.o, pf, cur_v, lane);
     };
 
-    int u = u_lo;
-    while (u < u_hi) {
+    int u = u0;
+    int seg_hi = u_hi;           // end of the ascending segment being walked
+    bool wrapped = (u0 == u_lo);  // the second segment [u_lo, u0) is under way (or empty)
+    while (true) {
         const TileClass tc = classify<MODE>(rules, m0, m1, u * kBN);
         // length of the run of tiles that use this same single pair with no mask (whole tiles, in range)
         int u_end = u;
         if (tc.fast) {
             u_end = u + 1;
-            while (u_end < u_hi) {
+            while (u_end < seg_hi) {
                 const TileClass t2 = classify<MODE>(rules, m0, m1, u_end * kBN);
                 if (!t2.fast || t2.main != tc.main) break;
                 ++u_end;
@@ -290,14 +306,20 @@ __global__ __launch_bounds__(kThreads, 2) void window_kernel(Params p) {
                     s[kb][r] = rules.visible(qi, j, qi_vis_lo) ? s[kb][r] : -INFINITY;
                 }
         }
-        if (u + 1 < u_hi) {
-            const int src = classify<MODE>(rules, m0, m1, n0 + kBN).main;
-            k_copy.load(nxt_k, k_ptr(src), k_stride(src), n0 + kBN, p.N);
-            v_copy.load(s_v[buf ^ 1], v_src, p.v.sn, n0 + kBN, p.N);
+        const int u_next = (u + 1 < seg_hi) ? u + 1 : (wrapped ? -1 : u_lo);
+        if (u_next >= 0) {
+            const int src = classify<MODE>(rules, m0, m1, u_next * kBN).main;
+            k_copy.load(nxt_k, k_ptr(src), k_stride(src), u_next * kBN, p.N);
+            v_copy.load(s_v[buf ^ 1], v_src, p.v.sn, u_next * kBN, p.N);
         }
         attend_tile(s, s_v[buf]);
         buf ^= 1;
-        ++u;
+        if (u_next < 0) break;
+        if (u_next != u + 1) {
+            wrapped = true;
+            seg_hi = u0;
+        }
+        u = u_next;
     }
 
     store_output<Tag, D>(st, p.out + b * p.o_sb + h * p.o_sh, p.o_sn,
