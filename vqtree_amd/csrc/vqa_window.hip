@@ -6,8 +6,9 @@
 //     pair B = (qb, kb)   keys beyond the window scored with the position-clamped query (ReRoPE)
 //     pair C = (qb, kc)   far keys replaced by their additive-quantiser reconstruction kc = sum_m codebook[m][code]
 // Tiles whose 128 x 64 (query x key) block uses a single pair and needs no mask take a fast path (one K tile,
-// prefetched a tile ahead); tiles on the diagonal, on the window edge or on the far-context boundary compute every
-// pair they touch and select / mask per element.
+// prefetched a tile ahead); tiles on the diagonal, on the window edge or on the far-context boundary are one step per
+// pair they touch (each wave scoring only the pairs its own 32 rows select, merged and masked per element), every
+// step's K tile requested one step ahead and the query operand of the next step requested behind the current product.
 #include "vqa_flash.h"
 
 namespace vqa {
@@ -37,6 +38,12 @@ struct Params {
     int pair_tiles;  // a workgroup handles query tiles (n-1-k, k) instead of one tile
     float scale_log2e;
 };
+
+// the value unchanged, but opaque to the optimiser: what is derived from it is not hoisted out of loops
+__device__ __forceinline__ int opaque(int x) {
+    asm volatile("" : "+v"(x));
+    return x;
+}
 
 __device__ __forceinline__ int floor_div(int a, int b) { return (a >= 0) ? a / b : -((-a + b - 1) / b); }
 
@@ -163,167 +170,246 @@ __global__ __launch_bounds__(kThreads, 2) void window_kernel(Params p) {
     k_copy.init(wave, lane);
     v_copy.init(wave, lane);
 
-    for (int pass = 0; pass < n_pass; ++pass) {
-    const int t = pass == 0 ? t_first : slot;
-    const int m0 = t * kBM;
-    const int m1 = min(m0 + kBM - 1, p.N - 1);
-    const int row0 = m0 + wave * 32;
-    const int qi = row0 + nq;  // this lane's query and its row bounds
-    const int qi_vis_lo = rules.vis_lo(qi);
-    const int qi_far_bnd = Rules<MODE>::kIsVq ? rules.far_bnd(qi) : 0;
-    if (pass) __syncthreads();  // the previous tile's last reads of the LDS buffers are done
-
-    // One query fragment set lives in registers: pair A's or pair B's.  Tiles are visited far -> near, so the
-    // operand in use changes O(1) times per workgroup; a change re-reads the wave's 32 rows (L2 hits).
     const uint16_t* qa_src = p.qa.p + b * p.qa.sb + h * p.qa.sh;
     const uint16_t* qb_src = p.qb.p + b * p.qb.sb + h * p.qb.sh;
-    QFrag<Tag, D> q;
-    int q_held = -1;
-    auto hold_q = [&](int which) {  // which: 0 = qa, 1 = qb (workgroup-uniform)
-        if (q_held != which) {
-            load_q<Tag, D>(q, which == 0 ? qa_src : qb_src, which == 0 ? p.qa.sn : p.qb.sn, row0, p.N, lane);
-            wait_tile_loads();  // settle the reload here so that later waits never have to cover it
-            q_held = which;
+    uint16_t* out_base = p.out + b * p.o_sb + h * p.o_sh;
+    float* lse_base = p.lse ? p.lse + (int64_t)bh * p.N : nullptr;
+
+    // The workgroup walks a flat list of STEPS: step = one (key tile, operand pair) score product.  A key tile that
+    // needs a single pair is one step; a tile on the window edge or the far-context boundary is one step per pair it
+    // touches, the products being merged per element.  The list runs over the key tiles of the first query tile,
+    // in the order given below, then over those of the second query tile (paired launch), so the loads of every step -- the
+    // first of a query tile included -- are requested one step ahead, and the K buffers alternate per step, the
+    // V buffers per key tile.  Within a tile the pair scored last in the previous tile goes first, which keeps the
+    // number of changes of the query operand per query tile at its minimum.
+    // Order of the key tiles of one query tile.  Modes that see the whole prefix walk up from key 0: the workgroups
+    // of one head start together and so read the same K / V tiles at about the same time, sharing them through
+    // the L2.  Sliding-window modes walk their window in a rotated order, key tile index modulo the number of
+    // tiles in a window -- [u0, u_hi) then [u_lo, u0) -- for the same reason: at any step the workgroups of
+    // neighbouring query tiles, which share most of their key tiles, are on tiles of the same residue.
+    constexpr bool kRotate = (MODE == kLocalStrict || MODE == kLocalLoose || MODE == kLocalRerope);
+    struct Cursor {
+        int pass, m0, m1, u, seg_hi, u_lo, u0, wrapped, valid;  // plain ints: the struct stays in scalar registers
+    };
+    auto open_pass = [&](int pass) __attribute__((always_inline)) {
+        Cursor c;
+        c.valid = pass < n_pass ? 1 : 0;
+        c.pass = pass;
+        const int t = pass == 0 ? t_first : slot;
+        c.m0 = t * kBM;
+        c.m1 = min(c.m0 + kBM - 1, p.N - 1);
+        const int hi_key = rules.is_causal() ? min(p.N, c.m1 + 1) : p.N;
+        c.seg_hi = (hi_key + kBN - 1) / kBN;
+        c.u_lo = max(0, rules.vis_lo(c.m0)) / kBN;
+        c.u0 = c.u_lo;
+        if (kRotate) {
+            const int period = (rules.W + kBM + kBN - 1) / kBN;
+            c.u0 = (c.u_lo + period - 1) / period * period;
+            if (c.u0 >= c.seg_hi) c.u0 = c.u_lo;
         }
+        c.u = c.u0;
+        c.wrapped = (c.u0 == c.u_lo) ? 1 : 0;
+        return c;
+    };
+    auto last_of_pass = [&](const Cursor& c) __attribute__((always_inline)) {
+        return c.u + 1 >= c.seg_hi && c.wrapped;
+    };
+    auto next_tile = [&](const Cursor& c) __attribute__((always_inline)) {
+        if (c.u + 1 < c.seg_hi) {
+            Cursor n = c;
+            ++n.u;
+            return n;
+        }
+        if (!c.wrapped) {
+            Cursor n = c;
+            n.u = c.u_lo;
+            n.seg_hi = c.u0;
+            n.wrapped = 1;
+            return n;
+        }
+        return open_pass(c.pass + 1);
+    };
+    // What one wave (32 query rows) has to do with a key tile, packed into one scalar: bits 0-2 the pairs that some
+    // element of the wave's 32 x 64 block selects, bit 3 "a single pair and nothing masked", bit 4 "some element
+    // is visible at all".
+    auto wave_tile = [&](const Cursor& c) __attribute__((always_inline)) {
+        const int r0 = min(c.m0 + wave * 32, p.N - 1), r1 = min(c.m0 + wave * 32 + 31, p.N - 1);
+        const int n0 = c.u * kBN;
+        const TileClass t = classify<MODE>(rules, r0, r1, n0);
+        const bool visible = (!rules.is_causal() || n0 <= r1) && (n0 + kBN - 1 >= rules.vis_lo(r0));
+        return t.need | (t.fast ? 8 : 0) | (visible ? 16 : 0);
+    };
+    auto wave_works = [](int tw, int src) __attribute__((always_inline)) { return (tw & 16) && ((tw >> src) & 1); };
+    // the workgroup-wide classification packed the same way: bits 0-2 pairs needed, bit 3 fast, bits 4-5 main pair
+    auto wg_tile = [&](const Cursor& c) __attribute__((always_inline)) {
+        const TileClass t = classify<MODE>(rules, c.m0, c.m1, c.u * kBN);
+        return t.need | (t.fast ? 8 : 0) | (t.main << 4);
+    };
+    auto first_src = [](int need, int prefer) __attribute__((always_inline)) {
+        return ((need >> prefer) & 1) ? prefer : __builtin_ctz(need);
+    };
+    auto next_src = [](int need, int done) __attribute__((always_inline)) {
+        const int rest = need & ~done;
+        return rest ? __builtin_ctz(rest) : -1;
     };
 
-    // key tiles this workgroup visits
-    const int hi_key = rules.is_causal() ? min(p.N, m1 + 1) : p.N;
-    const int u_hi = (hi_key + kBN - 1) / kBN;
-    const int u_lo = max(0, rules.vis_lo(m0)) / kBN;
-    // Sliding-window modes: neighbouring query tiles share most of their key tiles, and the workgroups of an XCD that
-    // run at the same time are neighbours.  If each started at its own first key tile, a key tile would be read by
-    // its (window / 128 + 1) users several steps apart, with megabytes of other tiles in between -- more than the L2
-    // holds, so it would come from memory again for each of them.  Instead every workgroup walks its window in the
-    // same rotated order, key tile index modulo the number of tiles in a window: at any step all of them are on
-    // tiles of the same residue, so the users of one tile read it at about the same time.  (The online softmax does
-    // not care about the order.)  The walk is [u0, u_hi) followed by [u_lo, u0).
-    constexpr bool kRotate = (MODE == kLocalStrict || MODE == kLocalLoose || MODE == kLocalRerope);
-    int u0 = u_lo;
-    if (kRotate) {
-        const int period = (rules.W + kBM + kBN - 1) / kBN;
-        u0 = (u_lo + period - 1) / period * period;
-        if (u0 >= u_hi) u0 = u_lo;
-    }
+    // One query fragment set lives in registers: pair A's or pair B's (pairs B and C share the query).
+    QFrag<Tag, D> q;
+    int q_held = -1;
+    auto q_id = [&](const Cursor& c, int src) __attribute__((always_inline)) {
+        return 2 * c.pass + ((kDual && src != 0) ? 1 : 0);
+    };
+    auto fetch_q = [&](const Cursor& c, int src) __attribute__((always_inline)) {
+        const bool second = kDual && src != 0;
+        load_q<Tag, D>(q, second ? qb_src : qa_src, second ? p.qb.sn : p.qa.sn, c.m0 + wave * 32, p.N, lane);
+        q_held = q_id(c, src);
+    };
 
     SoftmaxState<D> st;
     st.init();
 
-    int buf = 0;  // buffer holding the tile about to be computed: K of its main pair, and V
-    {
-        const int src = classify<MODE>(rules, m0, m1, u0 * kBN).main;
-        k_copy.load(s_k[0], k_ptr(src), k_stride(src), u0 * kBN, p.N);
-        v_copy.load(s_v[0], v_src, p.v.sn, u0 * kBN, p.N);
-    }
+    Cursor c = open_pass(0);
+    int tc = wg_tile(c);
+    int tw = wave_tile(c);
+    int src = first_src(tc & 7, tc >> 4);
+    int kbuf = 0, vbuf = 0;
+    k_copy.load(s_k[0], k_ptr(src), k_stride(src), c.u * kBN, p.N);
+    v_copy.load(s_v[0], v_src, p.v.sn, c.u * kBN, p.N);
+    if (wave_works(tw, src)) fetch_q(c, src);
 
-    // scores -> probabilities -> O update for the tile whose K / V sit in cur_k / cur_v
-    auto attend_tile = [&](f32x16_t(&s)[2], const char* cur_v) {
-        vec8 pf[2][2];
-        softmax_update<Tag, D, false>(st, s, p.scale_log2e, pf, nullptr);
-        pv_mma<Tag, D>(st.o, pf, cur_v, lane);
-    };
-
-    int u = u0;
-    int seg_hi = u_hi;           // end of the ascending segment being walked
-    bool wrapped = (u0 == u_lo);  // the second segment [u_lo, u0) is under way (or empty)
-    while (true) {
-        const TileClass tc = classify<MODE>(rules, m0, m1, u * kBN);
-        // length of the run of tiles that use this same single pair with no mask (whole tiles, in range)
-        int u_end = u;
-        if (tc.fast) {
-            u_end = u + 1;
-            while (u_end < seg_hi) {
-                const TileClass t2 = classify<MODE>(rules, m0, m1, u_end * kBN);
-                if (!t2.fast || t2.main != tc.main) break;
-                ++u_end;
+    while (c.valid) {
+        // A run of tiles that every wave scores with one pair and no mask goes through a loop of its own: nothing
+        // to classify per wave, whole-tile loads, one barrier per tile.  The last tile of a run is left to the
+        // general code below, which knows how to request whatever follows.
+        if (tc & 8) {
+            const int run_src = tc >> 4;
+            int run = 0;  // tiles after this one, contiguous in this segment, of the same kind
+            while (c.u + run + 1 < c.seg_hi) {
+                const TileClass t2 = classify<MODE>(rules, c.m0, c.m1, (c.u + run + 1) * kBN);
+                if (!t2.fast || t2.main != run_src) break;
+                ++run;
+            }
+            if (run > 0) {
+                if (q_held != q_id(c, run_src)) {
+                    wait_tile_loads();
+                    fetch_q(c, run_src);
+                    wait_tile_loads();
+                }
+                const uint16_t* run_k = k_ptr(run_src);
+                const int64_t run_sn = k_stride(run_src);
+                for (; run > 0; --run) {
+                    wait_tile_loads();
+                    __syncthreads();
+                    k_copy.load_full(s_k[kbuf ^ 1], run_k, run_sn, (c.u + 1) * kBN);
+                    v_copy.load_full(s_v[vbuf ^ 1], v_src, p.v.sn, (c.u + 1) * kBN);
+                    f32x16_t s[2];
+                    qk_mma<Tag, D>(s, q, s_k[kbuf], lane);
+                    vec8 pf[2][2];
+                    softmax_update<Tag, D, false>(st, s, p.scale_log2e, pf, nullptr);
+                    pv_mma<Tag, D>(st.o, pf, s_v[vbuf], lane);
+                    kbuf ^= 1;
+                    vbuf ^= 1;
+                    ++c.u;
+                }
+                tw = wave_tile(c);  // tc is unchanged: same kind of tile
             }
         }
-        if (u_end - u >= 2) {
-            // hot loop: tiles u .. u_end-2 (the run's last tile goes through the general path below, which also
-            // knows how to fetch whatever follows the run)
-            hold_q(kDual && tc.main != 0 ? 1 : 0);
-            const uint16_t* run_k = k_ptr(tc.main);
-            const int64_t run_sn = k_stride(tc.main);
-            for (; u < u_end - 1; ++u) {
-                wait_tile_loads();
-                __syncthreads();  // tile u is complete in `buf`; every wave is done with the other buffer
-                k_copy.load_full(s_k[buf ^ 1], run_k, run_sn, (u + 1) * kBN);
-                v_copy.load_full(s_v[buf ^ 1], v_src, p.v.sn, (u + 1) * kBN);
-                f32x16_t s[2];
-                qk_mma<Tag, D>(s, q, s_k[buf], lane);
-                attend_tile(s, s_v[buf]);
-                buf ^= 1;
-            }
+        const Cursor nc = next_tile(c);
+        int ntc = tc, ntw = tw;
+        if (nc.valid) {
+            ntc = wg_tile(nc);
+            ntw = wave_tile(nc);
         }
-
-        // general tile: every pair it touches, per-element selection and masking
-        const int n0 = u * kBN;
-        const TileClass tg = classify<MODE>(rules, m0, m1, n0);
-        const char* cur_k = s_k[buf];
-        const char* nxt_k = s_k[buf ^ 1];
-        wait_tile_loads();
-        __syncthreads();
+        const int n0 = c.u * kBN;
         f32x16_t s[2];
-        auto extra_pair = [&](int src) {  // pair `src` is scored in this tile besides the main one
-            if (MODE == kVqPrefill2 && src == 1) return false;
-            if (MODE != kVqPrefill && MODE != kVqPrefill2 && src == 2) return false;
-            return src != tg.main && ((tg.need >> src) & 1) != 0;
-        };
-        // the first extra pair's K tile is requested before the main product so that the product hides its latency
-        int early = -1;
-        if constexpr (kDual) {
-            early = extra_pair(0) ? 0 : (extra_pair(1) ? 1 : (extra_pair(2) ? 2 : -1));
-            if (early >= 0) k_copy.load(nxt_k, k_ptr(early), k_stride(early), n0, p.N);
-        }
-        hold_q(kDual && tg.main != 0 ? 1 : 0);
-        qk_mma<Tag, D>(s, q, cur_k, lane);
-        if constexpr (kDual) {
-            // the other pairs, one K tile at a time through the (still free) K buffer of the next tile
-            for (int src = 0; src < 3; ++src) {
-                if (!extra_pair(src)) continue;
-                if (src != early) k_copy.load(nxt_k, k_ptr(src), k_stride(src), n0, p.N);
-                hold_q(src == 0 ? 0 : 1);
+        bool have_s = false, first_step = true;
+        int done = 0, last_src = src;
+        while (src >= 0) {
+            done |= 1 << src;
+            last_src = src;
+            const int same = next_src(tc & 7, done);  // next pair of this tile, if any
+            const bool work = wave_works(tw, src);
+            wait_tile_loads();
+            __syncthreads();  // this step's K (and the tile's V) are complete; every wave is done with the last step
+            if (work && q_held != q_id(c, src)) {  // not requested ahead: this wave sat out the previous step
+                fetch_q(c, src);
                 wait_tile_loads();
-                __syncthreads();
+            }
+            // request what the next step reads
+            int f_src = same;
+            if (same >= 0) {
+                k_copy.load(s_k[kbuf ^ 1], k_ptr(same), k_stride(same), n0, p.N);
+            } else if (nc.valid) {
+                f_src = first_src(ntc & 7, src);
+                k_copy.load(s_k[kbuf ^ 1], k_ptr(f_src), k_stride(f_src), nc.u * kBN, p.N);
+            }
+            if (first_step && nc.valid) v_copy.load(s_v[vbuf ^ 1], v_src, p.v.sn, nc.u * kBN, p.N);
+            first_step = false;
+
+            if (work) {
+                if (!have_s) {
+                    qk_mma<Tag, D>(s, q, s_k[kbuf], lane);
+                    have_s = true;
+                } else {
+                    // per-lane row data is recomputed here (a few VALU operations) instead of living in registers
+                    // across the whole loop nest
+                    const int ln = opaque(lane);
+                    const int qi = c.m0 + wave * 32 + (ln & 31);
+                    const int qi_far_bnd = Rules<MODE>::kIsVq ? rules.far_bnd(qi) : 0;
 #pragma unroll
-                for (int kb = 0; kb < 2; ++kb) {
-                    const f32x16_t s2 = qk_block<Tag, D>(q, nxt_k, kb, lane);
+                    for (int kb = 0; kb < 2; ++kb) {
+                        const f32x16_t s2 = qk_block<Tag, D>(q, s_k[kbuf], kb, lane);
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        const int j = n0 + kb * 32 + key_of_reg(r, half);
-                        if (rules.source(qi, j, qi_far_bnd) == src) s[kb][r] = s2[r];
+                        for (int r = 0; r < 16; ++r) {
+                            const int j = n0 + kb * 32 + key_of_reg(r, ln >> 5);
+                            if (rules.source(qi, j, qi_far_bnd) == src) s[kb][r] = s2[r];
+                        }
                     }
                 }
-                __syncthreads();  // all waves have read this pair's K tile before the buffer is reused
             }
-        }
-        if (!tg.fast) {
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int j = n0 + kb * 32 + key_of_reg(r, half);
-                    s[kb][r] = rules.visible(qi, j, qi_vis_lo) ? s[kb][r] : -INFINITY;
+            // the query operand of the step after this one, if this wave takes part in it and holds the other one:
+            // requested now, behind the products that read the registers, so that the softmax and P.V hide it
+            if (f_src >= 0) {
+                __builtin_amdgcn_sched_barrier(0);  // keep the reload behind the products: one operand set in registers
+                const bool f_same = same >= 0;
+                const int fw = f_same ? tw : ntw;
+                if (wave_works(fw, f_src)) {
+                    if (f_same) {
+                        if (q_held != q_id(c, f_src)) fetch_q(c, f_src);
+                    } else {
+                        if (q_held != q_id(nc, f_src)) fetch_q(nc, f_src);
+                    }
                 }
+            }
+            kbuf ^= 1;
+            src = same;
         }
-        const int u_next = (u + 1 < seg_hi) ? u + 1 : (wrapped ? -1 : u_lo);
-        if (u_next >= 0) {
-            const int src = classify<MODE>(rules, m0, m1, u_next * kBN).main;
-            k_copy.load(nxt_k, k_ptr(src), k_stride(src), u_next * kBN, p.N);
-            v_copy.load(s_v[buf ^ 1], v_src, p.v.sn, u_next * kBN, p.N);
+        if (have_s) {
+            if (!(tw & 8)) {
+                const int ln = opaque(lane);
+                const int qi = c.m0 + wave * 32 + (ln & 31);
+                const int qi_vis_lo = rules.vis_lo(qi);
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int j = n0 + kb * 32 + key_of_reg(r, ln >> 5);
+                        s[kb][r] = rules.visible(qi, j, qi_vis_lo) ? s[kb][r] : -INFINITY;
+                    }
+            }
+            vec8 pf[2][2];
+            softmax_update<Tag, D, false>(st, s, p.scale_log2e, pf, nullptr);
+            pv_mma<Tag, D>(st.o, pf, s_v[vbuf], lane);
         }
-        attend_tile(s, s_v[buf]);
-        buf ^= 1;
-        if (u_next < 0) break;
-        if (u_next != u + 1) {
-            wrapped = true;
-            seg_hi = u0;
+        if (last_of_pass(c)) {  // last key tile of this query tile
+            store_output<Tag, D>(st, out_base, p.o_sn, lse_base, c.m0 + wave * 32, p.N, lane);
+            st.init();
         }
-        u = u_next;
-    }
-
-    store_output<Tag, D>(st, p.out + b * p.o_sb + h * p.o_sh, p.o_sn,
-                         p.lse ? p.lse + (int64_t)bh * p.N : nullptr, row0, p.N, lane);
+        vbuf ^= 1;
+        c = nc;
+        tc = ntc;
+        tw = ntw;
+        src = c.valid ? first_src(tc & 7, last_src) : -1;
     }
 }
 
