@@ -371,6 +371,40 @@ int vqa_rope_f16(const void* x, const int64_t* position_ids, const void* cos, co
                  void* out_fixed, int B, int H, int N, int D, int n_pos, int64_t table_stride, const int64_t* strides,
                  int fixed_pos, vqa_stream_t stream);
 
+/* ------------------------------------------------------------------------------------------------------------------
+ * Count state of a single-codebook key cache and the generation step over it.  With one codebook a quantised key IS a
+ * codeword, so attention over N quantised keys equals attention over the C codewords with weights:
+ *     sum_j exp(q.cb[id_j]) v_j = sum_c exp(q.cb[c]) Vsum[c],      Z = sum_c cnt[c] exp(q.cb[c]).
+ * (cnt, Vsum) is the state the reference's cache stores after a prefill -- key counts and cumulated values,
+ * ops/attn_vq.py:89-127 -- for the seqlen_q == 1 route it leaves unimplemented (ops/attn_vq.py:176-223, 445-479).
+ * A step costs O(C D) whatever the context length.
+ *
+ *   vqa_count_state_add: fold T keys into the state, cnt[b,h,ids[b,h,t]] += 1 and Vsum[b,h,ids[b,h,t],:] += v[b,h,t,:]
+ *     (fp32 sums in position order, no atomics: results are reproducible).  ids [B,H,T] int64 (entries outside [0, C)
+ *     are skipped), v [B,H,T,D]; cnt [B,H,C] int32 and vsum [B,H,C,D] fp32 contiguous, zeroed by the caller before the
+ *     first call.  strides[0..5] = ids(b,h,t) v(b,h,t).  D in {64, 128}.
+ *   vqa_count_decode: out[b,h,:] = sum_c e_c Vsum[b,h,c,:] / Z with e_c = exp(q[b,h].cb[h,c] * sm_scale) for the
+ *     codewords with cnt > 0; lse (nullable, [B,H] fp32) = log2 Z, -inf for an empty state (out = 0) -- the pair is an
+ *     attention state that vqa_merge_state_inplace combines with the state of an exact window.
+ *     q, out [B,H,D]; codebook [H,C,D]; strides[0..5] = q(b,h) codebook(h,c) out(b,h).  C <= VQA_COUNT_STATE_MAX_CODES.
+ * ------------------------------------------------------------------------------------------------------------------ */
+#define VQA_COUNT_STATE_MAX_CODES 8192
+#define VQA_COUNT_STATE_NUM_STRIDES 6
+
+int vqa_count_state_add_bf16(const int64_t* ids, const void* v, int32_t* cnt, float* vsum, int B, int H, int T, int D,
+                             int C, const int64_t* strides, vqa_stream_t stream);
+
+int vqa_count_state_add_f16(const int64_t* ids, const void* v, int32_t* cnt, float* vsum, int B, int H, int T, int D,
+                            int C, const int64_t* strides, vqa_stream_t stream);
+
+int vqa_count_decode_bf16(const void* q, const void* codebook, const int32_t* cnt, const float* vsum, void* out,
+                          float* lse, int B, int H, int C, int D, const int64_t* strides, float sm_scale,
+                          vqa_stream_t stream);
+
+int vqa_count_decode_f16(const void* q, const void* codebook, const int32_t* cnt, const float* vsum, void* out,
+                         float* lse, int B, int H, int C, int D, const int64_t* strides, float sm_scale,
+                         vqa_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

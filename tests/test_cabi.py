@@ -103,21 +103,27 @@ def test_static_scratch_decode_refuses_oversized_problem_on_the_host(lib):
     assert rc == -9 and b"static" in lib.vqa_strerror(rc)
 
 
-def test_generation_after_a_512_entry_prefill_raises_instead_of_restarting():
+def test_generation_step_is_recognised_after_any_prefill():
     """A cache that has recorded a prefill classifies the next seqlen_q == 1 call as a generation step whatever the
-    codebook size; with more than 256 entries (no uint8 codes) that step raises instead of attending over one token."""
+    codebook size (it must not restart as a one-token prefill); without a GPU that step fails loudly in the HIP
+    layer -- there is no CPU fallback."""
     import torch
 
     from vqtree_amd.ops import attn_vq as A
 
     H, C, D, N = 2, 512, 64, 700
     cache = A.VectorQuantizedReRoPECache(256, torch.zeros(H, C, D, dtype=torch.bfloat16))
-    A._remember(cache, 0, torch.randint(0, C, (1, H, N)), torch.zeros(1, H, N, D, dtype=torch.bfloat16), N)
-    assert cache.get_seq_length() == N and cache.seen_tokens == N and cache.key_codes[0].dtype == torch.int16
-    assert int(cache.key_codes[0].max()) > 255
+    assert cache.get_seq_length() == 0
+    cache.seq_lengths.append(N)
+    cache.decode_state.append(None)
+    assert cache.get_seq_length() == N
     one = torch.zeros(1, H, 1, D, dtype=torch.bfloat16)
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(Exception) as e:
         A.dispatch_attn(one, one, one, torch.tensor([[N]]), cache)
+    assert cache.get_seq_length() == N  # nothing was recorded as a fresh prefill
+    assert not isinstance(e.value, AssertionError)
+    with pytest.raises(AssertionError):
+        A.dispatch_attn(one, one, one, torch.tensor([[N]]), A.VectorQuantizedReRoPECache(256, cache.codebook, sphere=True))
 
 
 def test_ops_refuse_cpu_tensors():

@@ -79,14 +79,17 @@ def test_short_prefill_then_generation_steps():
     want, _ = oracle.local_attn(q1, k1, v, N, "strict")
     assert_close_16(out.view(B, N, H, D).transpose(1, 2), want, "short prefill")
     assert cache.get_seq_length(0) == N and cache.seen_tokens == N
+    all_ids, all_v = cache.key_codes[0].long(), v
     for step in range(3):
         qs, ks, vs = _states(B, H, 1, D, torch.bfloat16, 20 + step)
         o = A.dispatch_attn(qs, ks, vs, torch.full((B, 1), N + step, device="cuda"), cache)
         n_now = N + step + 1
         assert cache.get_seq_length(0) == n_now and o.shape == (B, 1, H * D)
+        all_ids = torch.cat([all_ids, A.quantize_ids(ks, cb).unsqueeze(-1)], dim=2)
+        all_v = torch.cat([all_v, vs], dim=2)
         cos, sin = A.rope_tables(D, W + 2, dtype=torch.bfloat16, device="cuda")
         q2 = qs * cos[W + 1] + A.rotate_half(qs) * sin[W + 1]
-        want, _ = oracle.attn_vq_decode(q2, cache.key_codes[0], cb.unsqueeze(1), cache.value_cache[0], 1 / math.sqrt(D))
+        want, _ = oracle.attn_vq_decode(q2, all_ids, cb.unsqueeze(1), all_v, 1 / math.sqrt(D))
         assert_close_16(o.view(B, 1, H, D).transpose(1, 2), want, f"generation step {step}")
 
 

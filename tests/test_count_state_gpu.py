@@ -1,0 +1,125 @@
+"""GPU tests of the count state of a single-codebook key cache (per-codeword key counts and value sums) and of the
+generation steps that run on it: the state against brute-force sums, the count-weighted codeword attention against the
+dense per-key oracle (with one codebook the two are the same function), and `dispatch_attn` generating after prefills
+with 512 codewords -- all keys coded against `oracle.attn_vq_decode`, and with an exact window against the last row of
+an oracle prefill over the same tokens."""
+import math
+
+import pytest
+import torch
+
+import oracle
+from tests.util import assert_close_16, assert_close_lse
+from vqtree_amd.ops import attn_vq as A
+from vqtree_amd.ops.count_state import CountState, count_decode
+
+pytestmark = pytest.mark.gpu
+
+
+def _randn(*shape, seed, dtype=torch.bfloat16, std=1.0):
+    return (torch.randn(*shape, generator=torch.Generator("cpu").manual_seed(seed)) * std).to(dtype).cuda()
+
+
+@pytest.mark.parametrize("D,dtype", [(128, torch.bfloat16), (64, torch.float16)])
+def test_state_add_matches_brute_force_sums(D, dtype):
+    print(f"count state: add D{D} {dtype}", flush=True)
+    B, H, C, T = 2, 3, 160, 777  # C not a multiple of the 16-codeword groups' count only by accident; T ragged
+    g = torch.Generator("cpu").manual_seed(11)
+    ids = torch.randint(0, C, (B, H, T), generator=g)
+    ids[0, 0, :50] = 7          # a heavily used codeword
+    ids[ids == 9] = 10          # and an unused one
+    v = _randn(B, H, T, D, seed=12, dtype=dtype)
+    st = CountState(B, H, C, D, "cuda")
+    st.add(ids[:, :, :300].cuda(), v[:, :, :300])
+    st.add(ids[:, :, 300:].cuda(), v[:, :, 300:])          # a second call accumulates
+    st.add(ids[:, :, :0].cuda(), v[:, :, :0])              # empty call: no-op
+    onehot = torch.nn.functional.one_hot(ids, C).double()  # [B,H,T,C]
+    want_cnt = onehot.sum(2).to(torch.int32)
+    want_sum = torch.einsum("bhtc,bhtd->bhcd", onehot, v.double().cpu())
+    assert torch.equal(st.cnt.cpu(), want_cnt)              # integer work: bit-exact
+    assert int(st.cnt[0, 0, 9]) == 0 and st.n_keys == T
+    assert torch.allclose(st.vsum.double().cpu(), want_sum, atol=1e-3, rtol=1e-5)  # fp32 sums of <= 777 16-bit values
+    # ids outside [0, C) are skipped, strided values are honoured
+    st2 = CountState(B, H, C, D, "cuda")
+    bad = ids.clone()
+    bad[:, :, ::5] = C + 3
+    bad[:, :, 1::5] = -1
+    v_bnhd = v.transpose(1, 2).contiguous().transpose(1, 2)  # [B,H,T,D] view of a [B,T,H,D] buffer
+    st2.add(bad.cuda(), v_bnhd)
+    keep = ((bad >= 0) & (bad < C))
+    oh2 = torch.nn.functional.one_hot(bad.clamp(0, C - 1), C).double() * keep[..., None]
+    assert torch.equal(st2.cnt.cpu(), oh2.sum(2).to(torch.int32))
+    assert torch.allclose(st2.vsum.double().cpu(), torch.einsum("bhtc,bhtd->bhcd", oh2, v.double().cpu()), atol=1e-3,
+                          rtol=1e-5)
+
+
+@pytest.mark.parametrize("D,dtype,C", [(128, torch.bfloat16, 512), (64, torch.float16, 128), (128, torch.bfloat16, 1024)])
+def test_count_decode_equals_per_key_attention(D, dtype, C):
+    """With one codebook, count-weighted attention over the codewords IS attention over the quantised keys."""
+    print(f"count state: decode D{D} C{C} {dtype}", flush=True)
+    B, H, N = 2, 4, 1500
+    ids = torch.randint(0, C // 2, (B, H, N), generator=torch.Generator("cpu").manual_seed(21))  # half the codewords unused
+    cb = _randn(H, C, D, seed=22, dtype=dtype, std=0.5)
+    v = _randn(B, H, N, D, seed=23, dtype=dtype)
+    q = _randn(B, H, 1, D, seed=24, dtype=dtype)
+    st = CountState(B, H, C, D, "cuda").add(ids.cuda(), v)
+    out, lse = count_decode(q, cb, st, return_lse=True)
+    want, want_lse = oracle.attn_vq_decode(q.cpu(), ids.unsqueeze(-1), cb.unsqueeze(1).cpu(), v.cpu(), 1 / math.sqrt(D))
+    assert_close_16(out, want, "count decode")
+    assert_close_lse(lse, want_lse)
+    # an empty state attends over nothing
+    o0, l0 = count_decode(q, cb, CountState(B, H, C, D, "cuda"), return_lse=True)
+    assert float(o0.float().abs().max()) == 0.0 and bool(torch.isinf(l0).all()) and bool((l0 < 0).all())
+
+
+def test_generation_after_a_512_codeword_prefill():
+    """`dispatch_attn` generates after a long prefill with 512 codewords: every step is dense softmax over ALL keys
+    seen so far, each replaced by its codeword, with the clamped query."""
+    print("count state: generation after C=512 prefill", flush=True)
+    B, H, N, D, W, C = 2, 4, 700, 128, 256, 512
+    q, k, v = (_randn(B, H, N, D, seed=30 + i) for i in range(3))
+    cb = _randn(H, C, D, seed=33)
+    pos = torch.arange(N, device="cuda").unsqueeze(0).expand(B, -1)
+    cache = A.VectorQuantizedReRoPECache(W, cb)
+    A.dispatch_attn(q, k, v, pos, cache)
+    assert cache.get_seq_length(0) == N and cache.key_codes[0].dtype == torch.int16
+    all_ids, all_v = cache.key_codes[0].long(), v
+    cos, sin = A.rope_tables(D, W + 2, dtype=torch.bfloat16, device="cuda")
+    for step in range(3):
+        qs, ks, vs = (_randn(B, H, 1, D, seed=40 + 3 * step + i) for i in range(3))
+        o = A.dispatch_attn(qs, ks, vs, torch.full((B, 1), N + step, device="cuda"), cache)
+        assert cache.get_seq_length(0) == N + step + 1 and cache.seen_tokens == N + step + 1 and o.shape == (B, 1, H * D)
+        all_ids = torch.cat([all_ids, A.quantize_ids(ks, cb).unsqueeze(-1)], dim=2)
+        all_v = torch.cat([all_v, vs], dim=2)
+        q2 = qs * cos[W + 1] + A.rotate_half(qs) * sin[W + 1]
+        want, _ = oracle.attn_vq_decode(q2.cpu(), all_ids.cpu(), cb.unsqueeze(1).cpu(), all_v.cpu(), 1 / math.sqrt(D))
+        assert_close_16(o.view(B, 1, H, D).transpose(1, 2), want, f"generation step {step}")
+
+
+@pytest.mark.parametrize("N", [638, 300])
+def test_generation_with_exact_window_equals_the_last_prefill_row(N):
+    """With `generation_exact_window` a step equals the last row of a prefill over the same tokens: exact window,
+    clamped-query strip, codewords below the 128-aligned far boundary.  N = 638 with window 256 puts the far boundary
+    at 256 and moves it to 384 at the third step (rows leave the buffers for the count state); N = 300 starts from
+    a short prefill with no far context at all."""
+    print(f"count state: exact-window generation N{N}", flush=True)
+    B, H, D, W, C = 1, 2, 128, 256, 512
+    steps = 4
+    q, k, v = (_randn(B, H, N + steps, D, seed=50 + i) for i in range(3))
+    cb = _randn(H, C, D, seed=53)
+    pos = torch.arange(N + steps, device="cuda").unsqueeze(0).expand(B, -1)
+    cache = A.VectorQuantizedReRoPECache(W, cb, generation_exact_window=True)
+    A.dispatch_attn(q[:, :, :N], k[:, :, :N], v[:, :, :N], pos[:, :N], cache)
+    ids = A.quantize_ids(k, cb)
+    q1, k1, q2 = A.rerope_operands(q, k, pos, W)
+    for step in range(steps):
+        t = N + step
+        o = A.dispatch_attn(q[:, :, t:t + 1], k[:, :, t:t + 1], v[:, :, t:t + 1], pos[:, t:t + 1], cache)
+        n = t + 1
+        want, _ = oracle.attn_vq_prefill(q1[:, :, :n].cpu(), ids[:, :, :n].unsqueeze(-1).cpu(), cb.unsqueeze(1).cpu(),
+                                         v[:, :, :n].cpu(), k_exact=k1[:, :, :n].cpu(), window_size=W,
+                                         q2=q2[:, :, :n].cpu(), k2=k[:, :, :n].cpu())
+        assert_close_16(o.view(B, 1, H, D).transpose(1, 2), want[:, :, -1:], f"exact-window generation step {step}")
+    st = cache.decode_state[0]
+    assert st.length == N + steps and st.base == max(0, (N + steps - 1 - W) // 128 * 128)
+    assert int(st.state.cnt.sum()) == B * H * st.base

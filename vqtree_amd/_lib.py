@@ -49,6 +49,10 @@ SIGNATURES = {
     "vqa_encode_keys_f16": (c_int, [_P] * 4 + [c_int] * 6 + [_STRIDES, c_int, c_int, _P]),
     "vqa_rope_bf16": (c_int, [_P] * 6 + [c_int] * 5 + [c_int64, _STRIDES, c_int, _P]),
     "vqa_rope_f16": (c_int, [_P] * 6 + [c_int] * 5 + [c_int64, _STRIDES, c_int, _P]),
+    "vqa_count_state_add_bf16": (c_int, [_P] * 4 + [c_int] * 5 + [_STRIDES, _P]),
+    "vqa_count_state_add_f16": (c_int, [_P] * 4 + [c_int] * 5 + [_STRIDES, _P]),
+    "vqa_count_decode_bf16": (c_int, [_P] * 6 + [c_int] * 4 + [_STRIDES, c_float, _P]),
+    "vqa_count_decode_f16": (c_int, [_P] * 6 + [c_int] * 4 + [_STRIDES, c_float, _P]),
     "vqa_preprocess_workspace_bytes": (c_size_t, [c_int] * 4),
     "vqa_preprocess_bf16": (c_int, [_P] * 7 + [c_size_t] + [c_int] * 5 + [_STRIDES, _P]),
     "vqa_preprocess_f16": (c_int, [_P] * 7 + [c_size_t] + [c_int] * 5 + [_STRIDES, _P]),

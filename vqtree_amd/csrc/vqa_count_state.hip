@@ -1,0 +1,247 @@
+// Count state of a single-codebook VQ key cache, and the generation step over it.
+//
+// With one codebook every quantised key IS a codeword, so attention over N quantised keys collapses to attention over
+// the C codewords with weights:  sum_j exp(q.cb[id_j]) v_j = sum_c exp(q.cb[c]) Vsum[c],  Z = sum_c cnt[c] exp(q.cb[c])
+// where cnt[c] = #{j : id_j = c} and Vsum[c] = sum of the values of those keys.  The state (cnt [B,H,C] int32,
+// Vsum [B,H,C,D] fp32) is what the reference's cache stores after a prefill (key counts and cumulated values,
+// ops/attn_vq.py:89-127); a generation step costs O(C D) whatever the context length.
+//
+//   count_state_add : fold T more keys (codeword ids and values) into the state, in position order (deterministic:
+//                     every (b, h, codeword) is owned by one workgroup, no atomics)
+//   count_decode    : one query per (b, h) against the state -> normalised output and base-2 log-sum-exp, ready to be
+//                     merged with the state of an exact window
+#include "vqa_common.h"
+
+namespace vqa {
+namespace count_state {
+
+constexpr int kCodesPerGroup = 16;  // codewords owned by one workgroup of count_state_add
+constexpr int kBatch = 4;           // value rows whose loads are in flight together
+
+// grid (C / 16 code groups, B*H), D threads: thread d owns element d of the group's 16 accumulators.
+template <typename Tag, int D>
+__global__ __launch_bounds__(D) void add_kernel(const int64_t* __restrict__ ids, const uint16_t* __restrict__ v,
+                                                int32_t* __restrict__ cnt, float* __restrict__ vsum, int H, int T, int C,
+                                                int64_t i_sb, int64_t i_sh, int64_t i_st, int64_t v_sb, int64_t v_sh,
+                                                int64_t v_st) {
+    constexpr int kWaves = D / kWave;
+    __shared__ int s_list[D];        // positions of the chunk's keys that belong to this group, in order
+    __shared__ int s_code[D];        // their codeword (0..15 within the group)
+    __shared__ int s_wave_n[kWaves];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int bh = blockIdx.y, b = bh / H, h = bh % H;
+    const int c0 = blockIdx.x * kCodesPerGroup;
+    const int64_t* my_ids = ids + b * i_sb + h * i_sh;
+    const uint16_t* my_v = v + b * v_sb + h * v_sh;
+
+    float acc[kCodesPerGroup];
+    int n[kCodesPerGroup];
+#pragma unroll
+    for (int c = 0; c < kCodesPerGroup; ++c) {
+        acc[c] = 0.f;
+        n[c] = 0;
+    }
+    for (int t0 = 0; t0 < T; t0 += D) {
+        // order-preserving compaction of the chunk's keys that belong to this group
+        const int t = t0 + tid;
+        const int64_t id = t < T ? my_ids[t * i_st] : -1;
+        const int64_t rel = id - c0;
+        const bool mine = rel >= 0 && rel < kCodesPerGroup && id < C;
+        const uint64_t mask = __builtin_amdgcn_ballot_w64(mine);
+        if (lane == 0) s_wave_n[wave] = __builtin_popcountll(mask);
+        __syncthreads();
+        int base = 0, total = 0;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) {
+            const int nw = s_wave_n[w];
+            if (w < wave) base += nw;
+            total += nw;
+        }
+        if (mine) {
+            const int slot = base + __builtin_popcountll(mask & ((uint64_t(1) << lane) - 1));
+            s_list[slot] = t;
+            s_code[slot] = (int)rel;
+        }
+        __syncthreads();
+        // thread d adds element d of every listed row, kBatch rows' loads in flight together
+        for (int i0 = 0; i0 < total; i0 += kBatch) {
+            float x[kBatch];
+            int code[kBatch];
+#pragma unroll
+            for (int j = 0; j < kBatch; ++j) {
+                const int i = min(i0 + j, total - 1);
+                code[j] = (i0 + j < total) ? s_code[i] : -1;
+                x[j] = Elem<Tag>::from_bits(my_v[(int64_t)s_list[i] * v_st + tid]);
+            }
+#pragma unroll
+            for (int j = 0; j < kBatch; ++j)
+#pragma unroll
+                for (int c = 0; c < kCodesPerGroup; ++c) {  // compile-time register index: no scratch
+                    if (code[j] == c) {
+                        acc[c] += x[j];
+                        n[c] += 1;
+                    }
+                }
+        }
+        __syncthreads();  // the lists are rewritten by the next chunk
+    }
+    const int n_codes = min(kCodesPerGroup, C - c0);
+#pragma unroll
+    for (int c = 0; c < kCodesPerGroup; ++c) {
+        if (c < n_codes && n[c] > 0) {
+            const int64_t row = (int64_t)bh * C + c0 + c;
+            vsum[row * D + tid] += acc[c];
+            if (tid == 0) cnt[row] += n[c];
+        }
+    }
+}
+
+// grid B*H, 256 threads.
+constexpr int kDecodeThreads = 256;
+
+template <typename Tag, int D>
+__global__ __launch_bounds__(kDecodeThreads) void decode_kernel(const uint16_t* __restrict__ q,
+                                                                const uint16_t* __restrict__ codebook,
+                                                                const int32_t* __restrict__ cnt,
+                                                                const float* __restrict__ vsum, uint16_t* __restrict__ out,
+                                                                float* __restrict__ lse, int H, int C, int64_t q_sb,
+                                                                int64_t q_sh, int64_t cb_sh, int64_t cb_sc, int64_t o_sb,
+                                                                int64_t o_sh, float scale_log2e) {
+    extern __shared__ float s_e[];  // C scores, then weights exp2(score - max) (0 for codewords with no key)
+    __shared__ uint32_t s_q[D / 2];
+    __shared__ float s_red[kDecodeThreads / kWave];
+    __shared__ float s_part[kDecodeThreads / (D / 4)][D];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int bh = blockIdx.x, b = bh / H, h = bh % H;
+    const uint16_t* my_q = q + b * q_sb + h * q_sh;
+    const uint16_t* my_cb = codebook + h * cb_sh;
+    const int32_t* my_cnt = cnt + (int64_t)bh * C;
+    const float* my_vsum = vsum + (int64_t)bh * C * D;
+
+    if (tid < D / 2) s_q[tid] = reinterpret_cast<const uint32_t*>(my_q)[tid];
+    __syncthreads();
+
+    // scores: one codeword per thread; the query is read from LDS at a wave-uniform address (broadcast)
+    float m = -INFINITY;
+    for (int c = tid; c < C; c += kDecodeThreads) {
+        const uint4* row = reinterpret_cast<const uint4*>(my_cb + (int64_t)c * cb_sc);
+        float s = 0.f;
+#pragma unroll
+        for (int i = 0; i < D / 8; ++i) {
+            const uint4 kx = row[i];
+            s = Elem<Tag>::dot2(kx.x, s_q[4 * i + 0], s);
+            s = Elem<Tag>::dot2(kx.y, s_q[4 * i + 1], s);
+            s = Elem<Tag>::dot2(kx.z, s_q[4 * i + 2], s);
+            s = Elem<Tag>::dot2(kx.w, s_q[4 * i + 3], s);
+        }
+        s *= scale_log2e;
+        s_e[c] = s;
+        if (my_cnt[c] > 0) m = fmaxf(m, s);
+    }
+    m = wave_max(m);
+    if (lane == 0) s_red[wave] = m;
+    __syncthreads();
+    m = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
+    __syncthreads();
+    float z = 0.f;
+    for (int c = tid; c < C; c += kDecodeThreads) {
+        const int n = my_cnt[c];
+        const float e = n > 0 ? fast_exp2(s_e[c] - m) : 0.f;
+        s_e[c] = e;
+        z += e * (float)n;
+    }
+    z = wave_sum(z);
+    if (lane == 0) s_red[wave] = z;
+    __syncthreads();
+    z = (s_red[0] + s_red[1]) + (s_red[2] + s_red[3]);
+
+    // out[d] = sum_c e_c Vsum[c][d]: D/4 lanes cover a row (16 bytes each), the groups of lanes take rows in turn
+    constexpr int kLanesPerRow = D / 4, kGroups = kDecodeThreads / kLanesPerRow;
+    const int g = tid / kLanesPerRow, dl = tid % kLanesPerRow;
+    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+    for (int c = g; c < C; c += kGroups) {
+        const float e = s_e[c];
+        if (e != 0.f) acc += e * *reinterpret_cast<const f32x4_t*>(my_vsum + (int64_t)c * D + dl * 4);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) s_part[g][dl * 4 + i] = acc[i];
+    __syncthreads();
+    if (tid < D) {
+        float o = 0.f;
+#pragma unroll
+        for (int gg = 0; gg < kGroups; ++gg) o += s_part[gg][tid];
+        const float inv = z > 0.f ? 1.f / z : 0.f;
+        out[b * o_sb + h * o_sh + tid] = Elem<Tag>::to_bits(o * inv);
+    }
+    if (tid == 0 && lse) lse[bh] = z > 0.f ? m + fast_log2(z) : -INFINITY;
+}
+
+template <typename Tag>
+int add(const int64_t* ids, const void* v, int32_t* cnt, float* vsum, int B, int H, int T, int D, int C,
+        const int64_t* st, hipStream_t stream) {
+    if (B <= 0 || H <= 0 || T < 0 || C <= 0) return VQA_ERR_BAD_SHAPE;
+    if (D != 64 && D != 128) return VQA_ERR_UNSUPPORTED_HEAD_DIM;
+    if (!ids || !v || !cnt || !vsum || !st) return VQA_ERR_NULL_POINTER;
+    if (T == 0) return VQA_OK;
+    if ((int64_t)B * H > 65535) return VQA_ERR_BAD_SHAPE;
+    const dim3 grid((C + kCodesPerGroup - 1) / kCodesPerGroup, B * H);
+    const uint16_t* vp = static_cast<const uint16_t*>(v);
+    if (D == 64)
+        hipLaunchKernelGGL((add_kernel<Tag, 64>), grid, dim3(64), 0, stream, ids, vp, cnt, vsum, H, T, C, st[0], st[1],
+                           st[2], st[3], st[4], st[5]);
+    else
+        hipLaunchKernelGGL((add_kernel<Tag, 128>), grid, dim3(128), 0, stream, ids, vp, cnt, vsum, H, T, C, st[0], st[1],
+                           st[2], st[3], st[4], st[5]);
+    return launch_status();
+}
+
+template <typename Tag>
+int decode(const void* q, const void* codebook, const int32_t* cnt, const float* vsum, void* out, float* lse, int B,
+           int H, int C, int D, const int64_t* st, float sm_scale, hipStream_t stream) {
+    if (B <= 0 || H <= 0 || C <= 0 || C > VQA_COUNT_STATE_MAX_CODES) return VQA_ERR_BAD_SHAPE;
+    if (D != 64 && D != 128) return VQA_ERR_UNSUPPORTED_HEAD_DIM;
+    if (!q || !codebook || !cnt || !vsum || !out || !st) return VQA_ERR_NULL_POINTER;
+    if (!aligned16(codebook) || (st[2] % 8) || (st[3] % 8) || (reinterpret_cast<uintptr_t>(q) & 3u) || (st[0] % 2) ||
+        (st[1] % 2) || !aligned16(vsum))
+        return VQA_ERR_MISALIGNED;
+    const uint16_t* qp = static_cast<const uint16_t*>(q);
+    const uint16_t* cb = static_cast<const uint16_t*>(codebook);
+    uint16_t* op = static_cast<uint16_t*>(out);
+    const size_t lds = (size_t)C * sizeof(float);
+    const float scale_log2e = sm_scale * kLog2e;
+    if (D == 64)
+        hipLaunchKernelGGL((decode_kernel<Tag, 64>), dim3(B * H), dim3(kDecodeThreads), lds, stream, qp, cb, cnt, vsum,
+                           op, lse, H, C, st[0], st[1], st[2], st[3], st[4], st[5], scale_log2e);
+    else
+        hipLaunchKernelGGL((decode_kernel<Tag, 128>), dim3(B * H), dim3(kDecodeThreads), lds, stream, qp, cb, cnt, vsum,
+                           op, lse, H, C, st[0], st[1], st[2], st[3], st[4], st[5], scale_log2e);
+    return launch_status();
+}
+
+}  // namespace count_state
+}  // namespace vqa
+
+extern "C" {
+
+int vqa_count_state_add_bf16(const int64_t* ids, const void* v, int32_t* cnt, float* vsum, int B, int H, int T, int D,
+                             int C, const int64_t* strides, vqa_stream_t stream) {
+    return vqa::count_state::add<vqa::bf16_tag>(ids, v, cnt, vsum, B, H, T, D, C, strides, stream);
+}
+int vqa_count_state_add_f16(const int64_t* ids, const void* v, int32_t* cnt, float* vsum, int B, int H, int T, int D,
+                            int C, const int64_t* strides, vqa_stream_t stream) {
+    return vqa::count_state::add<vqa::f16_tag>(ids, v, cnt, vsum, B, H, T, D, C, strides, stream);
+}
+int vqa_count_decode_bf16(const void* q, const void* codebook, const int32_t* cnt, const float* vsum, void* out,
+                          float* lse, int B, int H, int C, int D, const int64_t* strides, float sm_scale,
+                          vqa_stream_t stream) {
+    return vqa::count_state::decode<vqa::bf16_tag>(q, codebook, cnt, vsum, out, lse, B, H, C, D, strides, sm_scale,
+                                                   stream);
+}
+int vqa_count_decode_f16(const void* q, const void* codebook, const int32_t* cnt, const float* vsum, void* out,
+                         float* lse, int B, int H, int C, int D, const int64_t* strides, float sm_scale,
+                         vqa_stream_t stream) {
+    return vqa::count_state::decode<vqa::f16_tag>(q, codebook, cnt, vsum, out, lse, B, H, C, D, strides, sm_scale,
+                                                  stream);
+}
+
+}  // extern "C"

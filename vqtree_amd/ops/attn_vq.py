@@ -249,22 +249,32 @@ class AttentionMode(Enum):
 
 class VectorQuantizedReRoPECache:
     """Holds what the reference's cache of the same name configures (ops/attn_vq.py:31-52): the exact-window length,
-    the per-head codebook [H,C,D], the `sphere` flag and the attention mode; plus, after a prefill, the decode state
-    (single-codebook key codes [B,H,N,1] uint8 when C <= 256, and V) so that seqlen_q == 1 steps can run
-    `attn_vq_decode`."""
+    the per-head codebook [H,C,D], the `sphere` flag and the attention mode; plus, after a prefill, what its
+    `update_prefill` stores for the generation steps (ops/attn_vq.py:89-127): per-codeword key counts and value sums
+    (`count_state.CountState`), and -- with `generation_exact_window` -- the buffers of the last exact keys and values
+    (`count_state.GenerationWindow`).
 
-    def __init__(self, window_length, codebook, sphere=False, *, attention_mode=AttentionMode.SORT_BASED_LINEAR):
+    `generation_exact_window=False` (default): a seqlen_q == 1 step attends over ALL keys through their codewords with
+    the clamped query, the quantity `attn_vq_decode` computes over a code stream, here in O(C D) per step.
+    `generation_exact_window=True`: the step equals the last row of a prefill over the same tokens -- exact window,
+    clamped-query strip, codewords before the 128-aligned far boundary."""
+
+    def __init__(self, window_length, codebook, sphere=False, *, attention_mode=AttentionMode.SORT_BASED_LINEAR,
+                 generation_exact_window=False):
         assert codebook.shape[1] % 128 == 0
         self.window_length = window_length
         self.codebook = codebook
         self.sphere = sphere
         self.attention_mode = attention_mode
-        self.key_codes = []    # per layer: [B,H,N,1] uint8 (only when the codebook has <= 256 entries)
-        self.value_cache = []  # per layer: [B,H,N,D]
+        self.generation_exact_window = generation_exact_window
+        self.key_codes = []      # per layer: codeword ids of the prefill, [B,H,N,1] uint8 (int16 above 256 codewords)
+        self.value_cache = []    # per layer: the prefill's values [B,H,N,D]
+        self.decode_state = []   # per layer: CountState or GenerationWindow
+        self.seq_lengths = []    # per layer: tokens seen
         self.seen_tokens = 0
 
     def get_seq_length(self, layer_idx=0):
-        return 0 if len(self.value_cache) <= layer_idx else self.value_cache[layer_idx].shape[-2]
+        return 0 if len(self.seq_lengths) <= layer_idx else self.seq_lengths[layer_idx]
 
 
 def rotate_half(x):
@@ -415,7 +425,7 @@ def long_prefilling_sort_based_linear(query_states, key_states, value_states, po
     q1, k1, q2 = rerope_operands(query_states, key_states, position_ids, cache.window_length, rope_base)
     out = vq_attn_forward(q1, q2, k1, cache.codebook, cnt, key_states, value_states, v_vq, vi,
                           cache.window_length, softmax_scale=1 / math.sqrt(D))
-    _remember(cache, layer_idx, ids, value_states, N)
+    _remember(cache, layer_idx, ids, value_states, N, k1, key_states)
     return out.transpose(1, 2).contiguous().flatten(2)
 
 
@@ -430,20 +440,32 @@ def long_prefilling_per_key(query_states, key_states, value_states, position_ids
     out = attn_vq_prefill(q1, ids.to(torch.uint8).unsqueeze(-1), cache.codebook.unsqueeze(1), value_states,
                           k_exact=k1, window_size=cache.window_length, q2=q2, k2=key_states,
                           softmax_scale=1 / math.sqrt(D), schedule="per_key")
-    _remember(cache, layer_idx, ids, value_states, N)
+    _remember(cache, layer_idx, ids, value_states, N, k1, key_states)
     return out.transpose(1, 2).contiguous().flatten(2)
 
 
-def _remember(cache, layer_idx, ids, value_states, n_tokens):
-    """Record a prefill in the cache.  The values (and with them `get_seq_length`) are always recorded, so the next
-    seqlen_q == 1 call is recognised as a generation step whatever the codebook size; the key codes are kept as uint8
-    when the codebook has at most 256 entries (what `attn_vq_decode` streams), as int16 otherwise."""
+def _remember(cache, layer_idx, ids, value_states, n_tokens, k1, key_states):
+    """Record a prefill in the cache (what `update_prefill` keeps, ops/attn_vq.py:89-127): the sequence length, so
+    that the next seqlen_q == 1 call is recognised as a generation step; the codeword ids and values as given; and the
+    state the generation steps run on -- the count state over all keys, or, with `generation_exact_window`, the count
+    state below the far boundary of the next query plus the buffers of the exact keys above it."""
+    from .count_state import CountState, GenerationWindow
+
     if layer_idx == 0:
         cache.seen_tokens += n_tokens
-    if len(cache.value_cache) <= layer_idx:
-        code_dtype = torch.uint8 if cache.codebook.shape[1] <= 256 else torch.int16
+    if len(cache.seq_lengths) <= layer_idx:
+        B, H, _, D = value_states.shape
+        C = cache.codebook.shape[1]
+        code_dtype = torch.uint8 if C <= 256 else torch.int16
         cache.key_codes.append(ids.to(code_dtype).unsqueeze(-1).contiguous())
         cache.value_cache.append(value_states)
+        state = CountState(B, H, C, D, value_states.device)
+        if cache.generation_exact_window:
+            state = GenerationWindow(cache.window_length, k1, key_states, value_states, ids, n_tokens, state)
+        else:
+            state.add(ids, value_states)
+        cache.decode_state.append(state)
+        cache.seq_lengths.append(n_tokens)
 
 
 def long_prefilling_slow_reference_impl(query_states, key_states, value_states, position_ids, cache, layer_idx=0,
@@ -454,7 +476,7 @@ def long_prefilling_slow_reference_impl(query_states, key_states, value_states, 
     W = cache.window_length
     q1, k1, q2 = rerope_operands(query_states, key_states, position_ids, W, rope_base)
     k_hat, ids, _ = multi_head_single_quantize(key_states, cache.codebook)
-    _remember(cache, layer_idx, ids, value_states, N)
+    _remember(cache, layer_idx, ids, value_states, N, k1, key_states)
     scale = 1.0 / math.sqrt(D)
     output = torch.zeros_like(query_states, memory_format=torch.contiguous_format)
     for b in range(B):
@@ -482,6 +504,7 @@ def dispatch_attn(query_states, key_states, value_states, position_ids, cache, l
     from .triton_fused_local_attn import flash_attn_func as causal_window_attention
 
     B, H, q_len, D = query_states.shape
+    assert not cache.sphere, "Not implemented"  # as the reference's forward, ops/attn_vq.py:198
     is_prefilling = cache.get_seq_length(layer_idx) == 0
     if is_prefilling and q_len > cache.window_length + BLOCK_SIZE:
         if cache.attention_mode == AttentionMode.SORT_BASED_LINEAR:
@@ -496,21 +519,30 @@ def dispatch_attn(query_states, key_states, value_states, position_ids, cache, l
         out = causal_window_attention(q1.transpose(1, 2), k1.transpose(1, 2), value_states.transpose(1, 2), q_len,
                                       softmax_scale=1 / math.sqrt(D))
         ids = quantize_ids(key_states, cache.codebook)
-        _remember(cache, layer_idx, ids, value_states, q_len)
+        _remember(cache, layer_idx, ids, value_states, q_len, k1, key_states)
         return out.contiguous().flatten(2)
     assert q_len == 1, "Only support prefilling or generation"
-    if cache.key_codes[layer_idx].dtype != torch.uint8:
-        raise NotImplementedError(
-            "generation after a prefill needs a codebook of at most 256 entries (uint8 key codes); this cache holds "
-            f"{cache.codebook.shape[1]}")
-    # generation step: append the new key's code and value, then attend over all codes with the clamped query
+    # Generation step on the state the prefill left (the route the reference leaves unimplemented,
+    # ops/attn_vq.py:176-223): O(C D) per step, whatever the context length and the codebook size.
+    from .count_state import count_decode
+
+    W = cache.window_length
+    t = cache.seq_lengths[layer_idx]  # position of the new token
     ids = quantize_ids(key_states, cache.codebook)
-    cache.key_codes[layer_idx] = torch.cat([cache.key_codes[layer_idx], ids.to(torch.uint8).unsqueeze(-1)], dim=2)
-    cache.value_cache[layer_idx] = torch.cat([cache.value_cache[layer_idx], value_states], dim=2)
+    state = cache.decode_state[layer_idx]
+    scale = 1 / math.sqrt(D)
+    cos, sin = rope_tables(D, max(W + 2, t + 1) if cache.generation_exact_window else W + 2, rope_base,
+                           query_states.dtype, query_states.device)
+    q2 = apply_rope(query_states, cos, sin, W + 1)
+    if cache.generation_exact_window:
+        q1 = apply_rope(query_states, cos, sin, t)
+        k1 = apply_rope(key_states, cos, sin, t)
+        state.append(k1, key_states, value_states, ids)
+        out = state.attend(q1, q2, cache.codebook, scale)
+    else:
+        state.add(ids, value_states)
+        out = count_decode(q2, cache.codebook, state, softmax_scale=scale)
+    cache.seq_lengths[layer_idx] = t + 1
     if layer_idx == 0:
         cache.seen_tokens += 1
-    cos, sin = rope_tables(D, cache.window_length + 2, rope_base, query_states.dtype, query_states.device)
-    q2 = query_states * cos[cache.window_length + 1] + rotate_half(query_states) * sin[cache.window_length + 1]
-    out = attn_vq_decode(q2, cache.key_codes[layer_idx], cache.codebook.unsqueeze(1), cache.value_cache[layer_idx],
-                         softmax_scale=1 / math.sqrt(D))
     return out.transpose(1, 2).contiguous().flatten(2)
