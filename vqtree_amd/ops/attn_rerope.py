@@ -1,6 +1,6 @@
 """Caller of the full-context ReRoPE kernel: the key/value cache with decode-time re-rotation and the attention
-routing of the reference's ReRoPE module (ops/attn_rerope.py:19-288), without the transformers module plumbing
-(projections and o_proj stay with the model; states arrive as [B,H,N,D]).
+routing of the reference's ReRoPE module (ops/attn_rerope.py:19-288) on [B,H,N,D] states.  The transformers module
+around it (projections, o_proj, `use_rerope`) is `hf_llama.LlamaFlashAttention2ReRoPE`, reachable from here by name.
 """
 import math
 
@@ -29,6 +29,13 @@ class ReRoPECache:
 
     def get_usable_length(self, new_seq_length, layer_idx=0):
         return self.get_seq_length(layer_idx)
+
+    # what a transformers (5.x) model asks of a cache while it builds its (unused) causal mask
+    def get_query_offset(self, layer_idx=0):
+        return self.get_seq_length(layer_idx)
+
+    def get_mask_sizes(self, query_length, layer_idx=0):
+        return self.get_seq_length(layer_idx) + query_length, 0
 
     def get_max_length(self):
         return int(1e8)
@@ -109,3 +116,13 @@ def rerope_attn_forward(query_states, key_states, value_states, position_ids, ca
         return out.reshape(B, q_len, H * D).contiguous()
     out = attn_exact_decode(q, keys, values, softmax_scale=scale)
     return out.transpose(1, 2).reshape(B, q_len, H * D).contiguous()
+
+
+def __getattr__(name):
+    # `LlamaFlashAttention2ReRoPE` and `use_rerope` (ops/attn_rerope.py:116, 291) live in hf_llama and are imported on
+    # first use, so that the operators do not pay for importing transformers.
+    if name in ("LlamaFlashAttention2ReRoPE", "use_rerope"):
+        from . import hf_llama
+
+        return getattr(hf_llama, name)
+    raise AttributeError(f"module {__name__!r} has no attribute {name!r}")

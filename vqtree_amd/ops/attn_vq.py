@@ -276,6 +276,19 @@ class VectorQuantizedReRoPECache:
     def get_seq_length(self, layer_idx=0):
         return 0 if len(self.seq_lengths) <= layer_idx else self.seq_lengths[layer_idx]
 
+    def get_usable_length(self, new_seq_length, layer_idx=0):
+        return self.get_seq_length(layer_idx)
+
+    def get_max_length(self):
+        return int(1e8)  # "some safe number", ops/attn_vq.py:85-87
+
+    # what a transformers (5.x) model asks of a cache while it builds its (unused) causal mask
+    def get_query_offset(self, layer_idx=0):
+        return self.get_seq_length(layer_idx)
+
+    def get_mask_sizes(self, query_length, layer_idx=0):
+        return self.get_seq_length(layer_idx) + query_length, 0
+
 
 def rotate_half(x):
     half = x.shape[-1] // 2
@@ -546,3 +559,13 @@ def dispatch_attn(query_states, key_states, value_states, position_ids, cache, l
     if layer_idx == 0:
         cache.seen_tokens += 1
     return out.transpose(1, 2).contiguous().flatten(2)
+
+
+def __getattr__(name):
+    # The transformers modules (`LlamaFlashAttention2VectorQuantizedReRoPE`, `use_rerope`, ops/attn_vq.py:176, 482)
+    # live in hf_llama and are imported on first use, so that the operators do not pay for importing transformers.
+    if name in ("LlamaFlashAttention2VectorQuantizedReRoPE", "use_rerope"):
+        from . import hf_llama
+
+        return hf_llama.use_vq_rerope if name == "use_rerope" else getattr(hf_llama, name)
+    raise AttributeError(f"module {__name__!r} has no attribute {name!r}")
