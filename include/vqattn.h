@@ -213,6 +213,25 @@ int vqa_vqcount_merge_f16(const void* q2, const void* k_vq, const void* k_vq_cnt
                           void* out, float* lse, int B, int H, int N, int D, int C, const int64_t* strides, int window,
                           float sm_scale, vqa_stream_t stream);
 
+/* vqa_vqcount_fwd / vqa_vqcount_merge with the per-block key counts as exact integers (int64 [B,H,NT,C], the dtype in
+ * which the reference builds them, ops/attn_vq.py:352-353, before it casts them to the model dtype at :431 -- a cast
+ * that rounds bf16 counts above 256).  Same strides array; the k_vq_cnt strides count int64 elements. */
+int vqa_vqcount_fwd_icnt_bf16(const void* q2, const void* k_vq, const int64_t* k_vq_cnt, const void* v_vq,
+                              const int64_t* vi, void* out, float* lse, int B, int H, int N, int D, int C,
+                              const int64_t* strides, int window, float sm_scale, vqa_stream_t stream);
+
+int vqa_vqcount_fwd_icnt_f16(const void* q2, const void* k_vq, const int64_t* k_vq_cnt, const void* v_vq,
+                             const int64_t* vi, void* out, float* lse, int B, int H, int N, int D, int C,
+                             const int64_t* strides, int window, float sm_scale, vqa_stream_t stream);
+
+int vqa_vqcount_merge_icnt_bf16(const void* q2, const void* k_vq, const int64_t* k_vq_cnt, const void* v_vq,
+                                const int64_t* vi, void* out, float* lse, int B, int H, int N, int D, int C,
+                                const int64_t* strides, int window, float sm_scale, vqa_stream_t stream);
+
+int vqa_vqcount_merge_icnt_f16(const void* q2, const void* k_vq, const int64_t* k_vq_cnt, const void* v_vq,
+                               const int64_t* vi, void* out, float* lse, int B, int H, int N, int D, int C,
+                               const int64_t* strides, int window, float sm_scale, vqa_stream_t stream);
+
 /* ------------------------------------------------------------------------------------------------------------------
  * In-place merge of two attention states with base-2 log-sum-exp: m = max(s, s'), o <- (o 2^(s-m) + o' 2^(s'-m)) /
  * (2^(s-m) + 2^(s'-m)), s <- m + log2(2^(s-m) + 2^(s'-m)); a side with s = -inf is ignored.

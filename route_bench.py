@@ -42,12 +42,12 @@ def run(batch=1, heads=32, tokens=8192, head_dim=128, window=1024, codes=512, de
     pos = torch.arange(N, device=device).unsqueeze(0).expand(B, -1)
     q1, k1, q2 = A.rerope_operands(q, k, pos, W)
     ids = Q.quantize_ids(k, cb)
-    cnt, v_vq, vi = A.segmented_preprocess(ids, v, C)
+    cnt, v_vq, vi = A.segmented_preprocess(ids, v, C, want_int64_counts=True)
     out = {
         "workload": f"long prefill with VQ memory: batch {B}, {H} heads, {N} tokens, head_dim {D}, window {W}, "
                     f"{C} codewords per head, bf16",
         "encode_keys_us": _time(lambda: Q.quantize_ids(k, cb)),
-        "preprocess_us": _time(lambda: A.segmented_preprocess(ids, v, C)),
+        "preprocess_us": _time(lambda: A.segmented_preprocess(ids, v, C, want_int64_counts=True)),
         "rotary_operands_us": _time(lambda: A.rerope_operands(q, k, pos, W)),
         "vq_attn_forward_us": _time(lambda: vq_attn_forward(q1, q2, k1, cb, cnt, k, v, v_vq, vi, W)),
         "dispatch_attn_whole_us": _time(lambda: A.dispatch_attn(q, k, v, pos, A.VectorQuantizedReRoPECache(W, cb))),

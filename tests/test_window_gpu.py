@@ -235,6 +235,38 @@ def test_vq_attn_forward_reference_route(N, W, C, D):
     assert_close_16(out, want, "count route vs per-key")
 
 
+def test_count_route_with_exact_integer_counts():
+    """Counts above 256 are not representable in bf16 (the reference casts them to the model dtype,
+    ops/attn_vq.py:431); with int64 counts -- what the preprocessing builds -- the count route stays on the per-key
+    definition.  1792 keys on 4 used codewords: up to ~450 keys per codeword."""
+    _say("count route, integer counts")
+    N, W, C, D, H, B = 1792, 128, 128, 128, 2, 1
+    dtype = torch.bfloat16
+    q, k, v = (_randn(B, H, N, D, seed=70 + s, dtype=dtype) for s in range(3))
+    cb = _randn(H, C, D, seed=73, dtype=dtype)
+    cos, sin = oracle.rope_tables(D, N + W + 2)
+    pos = torch.arange(N)
+    q1, k1, q2 = oracle.apply_rope(q, cos, sin, pos), oracle.apply_rope(k, cos, sin, pos), oracle.apply_rope(q, cos, sin, W + 1)
+    ids = torch.randint(0, 4, (B, H, N), generator=torch.Generator("cpu").manual_seed(74))
+    cnt, v_vq, vi = oracle.sort_based_preprocess(ids, v, C, dtype=dtype)
+    assert cnt.dtype == torch.int64 and int(cnt.max()) > 256
+    assert not torch.equal(cnt.to(dtype).to(torch.int64), cnt)  # the cast to bf16 does round these counts
+    want, _ = oracle.attn_vq_prefill(q1, ids[..., None], cb[:, None], v, k_exact=k1, window_size=W, q2=q2, k2=k)
+    dev = lambda *ts: [t.cuda() for t in ts]
+    out = triton_fused_vq_attn.vq_attn_forward(*dev(q1, q2, k1, cb, cnt, k, v, v_vq, vi), W)
+    route = oracle.vq_attn_forward(q1, q2, k1, cb, cnt, k, v, v_vq, vi, W)
+    assert_close_16(out, route, "count route, int64 counts")
+    assert_close_16(out, want, "count route, int64 counts, vs per-key")
+    o2, l2 = triton_fused_vq_attn.vq_count_forward(*dev(q2, cb, cnt, v_vq, vi), W)
+    want_o, want_l = oracle.vq_count_forward(q2, cb, cnt, v_vq, vi, W)
+    assert_close_16(o2, want_o, "count kernel, int64 counts")
+    assert_close_lse(l2, want_l, atol=5e-3)
+    # the log-sum-exp is where rounded counts show: with bf16 counts it is off by up to log2(1 + 2^-8)
+    _, l2_rounded = triton_fused_vq_attn.vq_count_forward(*dev(q2, cb, cnt.to(dtype), v_vq, vi), W)
+    far = slice(W + 128, N)
+    assert (l2[:, :, far].cpu() - want_l[:, :, far]).abs().max() < (l2_rounded[:, :, far].cpu() - want_l[:, :, far]).abs().max()
+
+
 def test_count_kernel_and_merge_separately():
     N, W, C, D = 700, 128, 256, 128
     q1, q2, k1, k, k_hat, ids, cb, v, cnt, v_vq, vi = _count_route_case(N, W, C, D, B=2, dtype=torch.bfloat16)

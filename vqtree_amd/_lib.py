@@ -43,6 +43,10 @@ SIGNATURES = {
     "vqa_vqcount_fwd_f16": (c_int, [_P] * 7 + [c_int] * 5 + [_STRIDES, c_int, c_float, _P]),
     "vqa_vqcount_merge_bf16": (c_int, [_P] * 7 + [c_int] * 5 + [_STRIDES, c_int, c_float, _P]),
     "vqa_vqcount_merge_f16": (c_int, [_P] * 7 + [c_int] * 5 + [_STRIDES, c_int, c_float, _P]),
+    "vqa_vqcount_fwd_icnt_bf16": (c_int, [_P] * 7 + [c_int] * 5 + [_STRIDES, c_int, c_float, _P]),
+    "vqa_vqcount_fwd_icnt_f16": (c_int, [_P] * 7 + [c_int] * 5 + [_STRIDES, c_int, c_float, _P]),
+    "vqa_vqcount_merge_icnt_bf16": (c_int, [_P] * 7 + [c_int] * 5 + [_STRIDES, c_int, c_float, _P]),
+    "vqa_vqcount_merge_icnt_f16": (c_int, [_P] * 7 + [c_int] * 5 + [_STRIDES, c_int, c_float, _P]),
     "vqa_merge_state_inplace_bf16": (c_int, [_P] * 4 + [c_int] * 4 + [_STRIDES, _P]),
     "vqa_merge_state_inplace_f16": (c_int, [_P] * 4 + [c_int] * 4 + [_STRIDES, _P]),
     "vqa_encode_keys_bf16": (c_int, [_P] * 4 + [c_int] * 6 + [_STRIDES, c_int, c_int, _P]),

@@ -12,7 +12,8 @@ struct CountParams {
     View q;                 // q2 [B,H,N,D]
     const uint16_t* cb;     // [H,C,D]
     int64_t cb_sh, cb_sc;
-    const uint16_t* cnt;    // [B,H,NT,C] in the element type
+    const uint16_t* cnt;    // [B,H,NT,C] in the element type, or
+    const int64_t* cnt_i64;  // the same as exact integers (then cnt is null); same strides
     int64_t cnt_sb, cnt_sh, cnt_st;
     View vvq;               // [B,H,N+1,D]
     const int64_t* vi;      // [B,H,NT,C]
@@ -62,7 +63,9 @@ __global__ __launch_bounds__(kThreads, 2) void count_kernel(CountParams p) {
     const int t = blockIdx.x;
     const int row0 = first + t * kTile + wave * 32;
     const uint16_t* cb = p.cb + h * p.cb_sh;
-    const uint16_t* cnt = p.cnt + b * p.cnt_sb + h * p.cnt_sh + t * p.cnt_st;
+    const int64_t cnt_off = b * p.cnt_sb + h * p.cnt_sh + t * p.cnt_st;
+    const uint16_t* cnt = p.cnt + cnt_off;
+    const int64_t* cnt_i64 = p.cnt_i64 ? p.cnt_i64 + cnt_off : nullptr;
     const int64_t* vi = p.vi + b * p.vi_sb + h * p.vi_sh + t * p.vi_st;
     const uint16_t* vvq = p.vvq.p + b * p.vvq.sb + h * p.vvq.sh;
 
@@ -83,7 +86,9 @@ __global__ __launch_bounds__(kThreads, 2) void count_kernel(CountParams p) {
     float cnt_f = 0.f;
     auto fetch_meta = [&](int c0) {
         v_copy.fetch_rows(rows, vi, c0, p.C, p.N);  // v_vq has N + 1 rows
-        cnt_f = (tid < kBN && c0 + tid < p.C) ? Elem<Tag>::from_bits(cnt[c0 + tid]) : 0.f;  // 0: masked
+        cnt_f = 0.f;  // 0: masked
+        if (tid < kBN && c0 + tid < p.C)
+            cnt_f = cnt_i64 ? (float)cnt_i64[c0 + tid] : Elem<Tag>::from_bits(cnt[c0 + tid]);
     };
     auto request = [&](int c0, int buf) {  // uses the metadata fetched for c0
         k_copy.load(s_k[buf], cb, p.cb_sc, c0, p.C);
@@ -179,7 +184,7 @@ int launch_count(const CountParams& p, dim3 grid, hipStream_t stream) {
 template <typename Tag>
 int vqcount(const void* q2, const void* k_vq, const void* k_vq_cnt, const void* v_vq, const int64_t* vi, void* out,
             float* lse, int B, int H, int N, int D, int C, const int64_t* strides, int window, float sm_scale,
-            bool merge_into, hipStream_t stream) {
+            bool merge_into, bool integer_counts, hipStream_t stream) {
     if (!q2 || !k_vq || !k_vq_cnt || !v_vq || !vi || !out || !strides) return VQA_ERR_NULL_POINTER;
     if (merge_into && !lse) return VQA_ERR_NULL_POINTER;
     if (B <= 0 || H <= 0 || N <= 0 || C <= 0) return VQA_ERR_BAD_SHAPE;
@@ -189,7 +194,8 @@ int vqcount(const void* q2, const void* k_vq, const void* k_vq_cnt, const void* 
     p.q = View{static_cast<const uint16_t*>(q2), strides[0], strides[1], strides[2]};
     p.cb = static_cast<const uint16_t*>(k_vq);
     p.cb_sh = strides[3], p.cb_sc = strides[4];
-    p.cnt = static_cast<const uint16_t*>(k_vq_cnt);
+    p.cnt = integer_counts ? nullptr : static_cast<const uint16_t*>(k_vq_cnt);
+    p.cnt_i64 = integer_counts ? static_cast<const int64_t*>(k_vq_cnt) : nullptr;
     p.cnt_sb = strides[5], p.cnt_sh = strides[6], p.cnt_st = strides[7];
     p.vvq = View{static_cast<const uint16_t*>(v_vq), strides[8], strides[9], strides[10]};
     p.vi = vi;
@@ -307,28 +313,56 @@ int vqa_vqcount_fwd_bf16(const void* q2, const void* k_vq, const void* k_vq_cnt,
                          void* out, float* lse, int B, int H, int N, int D, int C, const int64_t* strides, int window,
                          float sm_scale, vqa_stream_t stream) {
     return vqa::flash::vqcount<vqa::bf16_tag>(q2, k_vq, k_vq_cnt, v_vq, vi, out, lse, B, H, N, D, C, strides, window,
-                                              sm_scale, false, stream);
+                                              sm_scale, false, false, stream);
 }
 
 int vqa_vqcount_fwd_f16(const void* q2, const void* k_vq, const void* k_vq_cnt, const void* v_vq, const int64_t* vi,
                         void* out, float* lse, int B, int H, int N, int D, int C, const int64_t* strides, int window,
                         float sm_scale, vqa_stream_t stream) {
     return vqa::flash::vqcount<vqa::f16_tag>(q2, k_vq, k_vq_cnt, v_vq, vi, out, lse, B, H, N, D, C, strides, window,
-                                             sm_scale, false, stream);
+                                             sm_scale, false, false, stream);
 }
 
 int vqa_vqcount_merge_bf16(const void* q2, const void* k_vq, const void* k_vq_cnt, const void* v_vq, const int64_t* vi,
                            void* out, float* lse, int B, int H, int N, int D, int C, const int64_t* strides,
                            int window, float sm_scale, vqa_stream_t stream) {
     return vqa::flash::vqcount<vqa::bf16_tag>(q2, k_vq, k_vq_cnt, v_vq, vi, out, lse, B, H, N, D, C, strides, window,
-                                              sm_scale, true, stream);
+                                              sm_scale, true, false, stream);
 }
 
 int vqa_vqcount_merge_f16(const void* q2, const void* k_vq, const void* k_vq_cnt, const void* v_vq, const int64_t* vi,
                           void* out, float* lse, int B, int H, int N, int D, int C, const int64_t* strides, int window,
                           float sm_scale, vqa_stream_t stream) {
     return vqa::flash::vqcount<vqa::f16_tag>(q2, k_vq, k_vq_cnt, v_vq, vi, out, lse, B, H, N, D, C, strides, window,
-                                             sm_scale, true, stream);
+                                             sm_scale, true, false, stream);
+}
+
+int vqa_vqcount_fwd_icnt_bf16(const void* q2, const void* k_vq, const int64_t* k_vq_cnt, const void* v_vq,
+                              const int64_t* vi, void* out, float* lse, int B, int H, int N, int D, int C,
+                              const int64_t* strides, int window, float sm_scale, vqa_stream_t stream) {
+    return vqa::flash::vqcount<vqa::bf16_tag>(q2, k_vq, k_vq_cnt, v_vq, vi, out, lse, B, H, N, D, C, strides, window,
+                                              sm_scale, false, true, stream);
+}
+
+int vqa_vqcount_fwd_icnt_f16(const void* q2, const void* k_vq, const int64_t* k_vq_cnt, const void* v_vq,
+                             const int64_t* vi, void* out, float* lse, int B, int H, int N, int D, int C,
+                             const int64_t* strides, int window, float sm_scale, vqa_stream_t stream) {
+    return vqa::flash::vqcount<vqa::f16_tag>(q2, k_vq, k_vq_cnt, v_vq, vi, out, lse, B, H, N, D, C, strides, window,
+                                             sm_scale, false, true, stream);
+}
+
+int vqa_vqcount_merge_icnt_bf16(const void* q2, const void* k_vq, const int64_t* k_vq_cnt, const void* v_vq,
+                                const int64_t* vi, void* out, float* lse, int B, int H, int N, int D, int C,
+                                const int64_t* strides, int window, float sm_scale, vqa_stream_t stream) {
+    return vqa::flash::vqcount<vqa::bf16_tag>(q2, k_vq, k_vq_cnt, v_vq, vi, out, lse, B, H, N, D, C, strides, window,
+                                              sm_scale, true, true, stream);
+}
+
+int vqa_vqcount_merge_icnt_f16(const void* q2, const void* k_vq, const int64_t* k_vq_cnt, const void* v_vq,
+                               const int64_t* vi, void* out, float* lse, int B, int H, int N, int D, int C,
+                               const int64_t* strides, int window, float sm_scale, vqa_stream_t stream) {
+    return vqa::flash::vqcount<vqa::f16_tag>(q2, k_vq, k_vq_cnt, v_vq, vi, out, lse, B, H, N, D, C, strides, window,
+                                             sm_scale, true, true, stream);
 }
 
 int vqa_merge_state_inplace_bf16(void* o, float* s, const void* o_other, const float* s_other, int B, int H, int N,

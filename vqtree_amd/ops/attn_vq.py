@@ -175,7 +175,7 @@ def attn_vq_prefill(q, k_codes, codebooks, v, *, k_exact=None, window_size=0, ca
         from .triton_fused_vq_attn import vq_attn_forward
 
         ids = k_codes[..., 0].to(torch.int64)
-        cnt, v_vq, vi = segmented_preprocess(ids, v, K)
+        cnt, v_vq, vi = segmented_preprocess(ids, v, K, want_int64_counts=True)
         return vq_attn_forward(q, q if q2 is None else q2, k_exact, codebooks[:, 0], cnt,
                                k_exact if (q2 is None or k2 is None) else k2, v, v_vq, vi, window_size,
                                softmax_scale=softmax_scale, return_lse=return_lse)
@@ -434,7 +434,7 @@ def long_prefilling_sort_based_linear(query_states, key_states, value_states, po
     B, H, N, D = query_states.shape
     dtype = query_states.dtype
     ids = quantize_ids(key_states, cache.codebook)
-    cnt, v_vq, vi = segmented_preprocess(ids, value_states, cache.codebook.shape[1])
+    cnt, v_vq, vi = segmented_preprocess(ids, value_states, cache.codebook.shape[1], want_int64_counts=True)
     q1, k1, q2 = rerope_operands(query_states, key_states, position_ids, cache.window_length, rope_base)
     out = vq_attn_forward(q1, q2, k1, cache.codebook, cnt, key_states, value_states, v_vq, vi,
                           cache.window_length, softmax_scale=1 / math.sqrt(D))

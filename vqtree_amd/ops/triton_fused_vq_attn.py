@@ -30,7 +30,8 @@ def _count_call(q2, k_vq, k_vq_cnt, v_vq, vi, window_size, softmax_scale, out, l
     _lib.require_gpu(q2, k_vq, k_vq_cnt, v_vq, vi)
     B, H, N, D = q2.shape
     C = k_vq.shape[1]
-    sfx = check_same_16bit(q2, k_vq, k_vq_cnt, v_vq)
+    integer_counts = k_vq_cnt.dtype == torch.int64  # exact counts, as the preprocessing builds them
+    sfx = check_same_16bit(q2, k_vq, None if integer_counts else k_vq_cnt, v_vq)
     assert vi.dtype == torch.int64 and k_vq.shape == (H, C, D) and v_vq.shape[:2] == (B, H)
     assert k_vq_cnt.shape[-1] == C and vi.shape == k_vq_cnt.shape
     n_far = max(0, -(-(N - window_size - 128) // 128))
@@ -38,7 +39,8 @@ def _count_call(q2, k_vq, k_vq_cnt, v_vq, vi, window_size, softmax_scale, out, l
     strides = _lib.strides_array(*bhn_strides(q2), k_vq.stride(0), k_vq.stride(1), *bhn_strides(k_vq_cnt),
                                  *bhn_strides(v_vq), *bhn_strides(vi), *bhn_strides(out))
     with torch.cuda.device(q2.device):
-        rc = getattr(lib, ("vqa_vqcount_merge_" if merge else "vqa_vqcount_fwd_") + sfx)(
+        name = ("vqa_vqcount_merge_" if merge else "vqa_vqcount_fwd_") + ("icnt_" if integer_counts else "")
+        rc = getattr(lib, name + sfx)(
             ptr(q2), ptr(k_vq), ptr(k_vq_cnt), ptr(v_vq), ptr(vi), ptr(out), ptr(lse), B, H, N, D, C, strides,
             int(window_size), softmax_scale, _lib.current_stream(q2.device))
     _lib.check(rc)
@@ -57,7 +59,8 @@ def vq_count_forward(q2, k_vq, k_vq_cnt, v_vq, vi, window_size, softmax_scale=No
 
 def vq_attn_forward(q1, q2, k1, k_vq, k_vq_cnt, k3, v, v_vq, vi, window_size, softmax_scale=None, return_lse=False):
     """q1/k1: rotary at true positions; q2: query at the clamped position; k_vq [H,C,D] codebook; k_vq_cnt / vi
-    [B,H,N//128,C] running counts / prefix-sum row indices sampled per 128-key block; k3 raw keys; v_vq [B,H,N+1,D]
+    [B,H,N//128,C] running counts (model dtype as in the reference, or int64 for exact counts -- bf16 rounds counts
+    above 256) / prefix-sum row indices sampled per 128-key block; k3 raw keys; v_vq [B,H,N+1,D]
     per-code prefix sums of V.  All attention tensors [B,H,N,D].  Returns [B,H,N,D] (with `return_lse`, an extension,
     also the merged base-2 log-sum-exp [B,H,N]).
 
