@@ -154,13 +154,28 @@ int vqa_prefill_f16(const void* q, const uint8_t* codes, const void* codebooks, 
                     int B, int H, int N, int D, int M, int K, const int64_t* strides, int window, int boundary_mode,
                     int causal, float sm_scale, vqa_stream_t stream);
 
-/* The same prefill on the software-pipelined schedule (one wave per SIMD with 64 query rows, the exponentials of a key
- * tile evaluated under the score MFMAs of the next one), for the reference's long-prefill configuration only: no second
- * query / key pair, the block boundary rule, `window` a multiple of 128 (or k_exact == NULL: every key quantised).
- * Anything else returns VQA_ERR_BAD_ARGUMENT.  Same strides array as vqa_prefill_* (the q2 / k2 slots are ignored), same
- * workspace, same results within the 16-bit tolerance; on MI355X it runs level with vqa_prefill_* and is kept as the
- * starting point for a schedule that overlaps softmax and matrix work inside one wave.  Counterpart in the reference: the
- * two launches of ops/triton_fused_vq_attn.py:202-245. */
+/* vqa_prefill_* picks between two schedules of the fused kernel:
+ *   tiled     -- 128-row query tiles, two workgroups per CU, every combination of arguments;
+ *   pipelined -- 256-row query tiles, one wave per SIMD with 64 query rows, the exponentials of a key tile evaluated
+ *                under the score MFMAs of the next one; only for the reference's long-prefill configuration: no
+ *                second query / key pair, the block boundary rule, `window` a multiple of 128 (or k_exact == NULL:
+ *                every key quantised).
+ * It takes the pipelined one where that is measurably faster on MI355X (3 - 7 %): when it applies, D == 128,
+ * N >= 4096 and the launch has at least 512 workgroups (two rounds for the 256 CUs).  The two entry points below force
+ * a schedule: vqa_prefill_tiled_* has vqa_prefill_*'s signature; vqa_prefill_pipelined_* returns VQA_ERR_BAD_ARGUMENT
+ * where the pipelined schedule does not apply (same strides array, the q2 / k2 slots are ignored).  Same workspace,
+ * same results within the 16-bit tolerance.  Counterpart in the reference: the two launches of
+ * ops/triton_fused_vq_attn.py:202-245. */
+int vqa_prefill_tiled_bf16(const void* q, const uint8_t* codes, const void* codebooks, const void* v,
+                           const void* k_exact, const void* q2, const void* k2, void* out, float* lse, void* workspace,
+                           size_t workspace_bytes, int B, int H, int N, int D, int M, int K, const int64_t* strides,
+                           int window, int boundary_mode, int causal, float sm_scale, vqa_stream_t stream);
+
+int vqa_prefill_tiled_f16(const void* q, const uint8_t* codes, const void* codebooks, const void* v,
+                          const void* k_exact, const void* q2, const void* k2, void* out, float* lse, void* workspace,
+                          size_t workspace_bytes, int B, int H, int N, int D, int M, int K, const int64_t* strides,
+                          int window, int boundary_mode, int causal, float sm_scale, vqa_stream_t stream);
+
 int vqa_prefill_pipelined_bf16(const void* q, const uint8_t* codes, const void* codebooks, const void* v,
                                const void* k_exact, void* out, float* lse, void* workspace, size_t workspace_bytes,
                                int B, int H, int N, int D, int M, int K, const int64_t* strides, int window, int causal,

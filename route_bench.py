@@ -17,10 +17,11 @@ if ROOT not in sys.path:
 
 from vqtree_amd.ops import attn_vq as A  # noqa: E402
 from vqtree_amd.ops import mini_vq as Q  # noqa: E402
+from vqtree_amd.ops.count_state import CountState  # noqa: E402
 from vqtree_amd.ops.triton_fused_vq_attn import vq_attn_forward  # noqa: E402
 
 
-def _time(fn, steps=10, warmup=3):
+def _time(fn, steps=20, warmup=10):
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
@@ -50,6 +51,7 @@ def run(batch=1, heads=32, tokens=8192, head_dim=128, window=1024, codes=512, de
         "preprocess_us": _time(lambda: A.segmented_preprocess(ids, v, C, want_int64_counts=True)),
         "rotary_operands_us": _time(lambda: A.rerope_operands(q, k, pos, W)),
         "vq_attn_forward_us": _time(lambda: vq_attn_forward(q1, q2, k1, cb, cnt, k, v, v_vq, vi, W)),
+        "count_state_build_us": _time(lambda: CountState(B, H, C, D, device).add(ids, v)),
         "dispatch_attn_whole_us": _time(lambda: A.dispatch_attn(q, k, v, pos, A.VectorQuantizedReRoPECache(W, cb))),
     }
     # the same attention through the fused per-key kernel (needs uint8 codes: at most 256 codewords)
@@ -60,6 +62,14 @@ def run(batch=1, heads=32, tokens=8192, head_dim=128, window=1024, codes=512, de
                                   schedule="per_key"))
     out["attn_vq_prefill_default_256_codewords_us"] = _time(  # M = 1: dispatched to the codeword-space route
         lambda: A.attn_vq_prefill(q1, ids256, cb256.unsqueeze(1), v, k_exact=k1, window_size=W, q2=q2, k2=k))
+    # the four-codebook prefill benchmark workload under the two schedules of the fused kernel
+    from vqtree_amd.synthetic import prefill_c3
+
+    c = prefill_c3()
+    for schedule in ("default", "pipelined"):
+        out[f"attn_vq_prefill_4x256_{schedule}_us"] = _time(
+            lambda: A.attn_vq_prefill(c.q, c.codes, c.codebooks, c.v, k_exact=c.k_exact, window_size=c.window,
+                                      softmax_scale=c.softmax_scale, schedule=schedule))
     return out
 
 

@@ -368,6 +368,34 @@ def test_vq_prefill_pipelined_schedule(B, H, N, D, M, W, dtype):
     assert (out.float() - ref.float()).abs().max() <= 2e-2
 
 
+def test_vq_prefill_schedule_choice_at_a_large_shape():
+    """64 heads x 4096 tokens (512 workgroups of 256 query rows in pairs): vqa_prefill_* takes the pipelined schedule
+    here.  The default call must be bit-identical to the forced pipelined one, within tolerance of the forced tiled
+    one, and two heads are checked against the oracle (heads are independent)."""
+    _say("vq prefill schedule choice H64 N4096")
+    B, H, N, D, M, W = 1, 64, 4096, 128, 4, 1024
+    g = torch.Generator(device="cuda").manual_seed(97)
+    q, k, v = (torch.randn(B, H, N, D, generator=g, device="cuda").to(torch.bfloat16) for _ in range(3))
+    cb = (torch.randn(H, M, 256, D, generator=g, device="cuda") * 0.35).to(torch.bfloat16)
+    codes = torch.randint(0, 256, (B, H, N, M), generator=g, device="cuda", dtype=torch.uint8)
+    run = lambda schedule: attn_vq_prefill(q, codes, cb, v, k_exact=k, window_size=W, return_lse=True, schedule=schedule)
+    (auto, auto_l), (tiled, tiled_l), (piped, piped_l) = run("default"), run("tiled"), run("pipelined")
+    torch.cuda.synchronize()
+    assert torch.equal(auto, piped) and torch.equal(auto_l, piped_l)
+    assert not torch.equal(auto, tiled)  # two kernels, two summation orders
+    assert (auto.float() - tiled.float()).abs().max() <= 2e-2
+    hs = [0, 37]
+    want, want_l = oracle.attn_vq_prefill(q[:, hs].cpu(), codes[:, hs].cpu(), cb[hs].cpu(), v[:, hs].cpu(),
+                                          k_exact=k[:, hs].cpu(), window_size=W)
+    assert_close_16(auto[:, hs], want, "auto schedule")
+    assert_close_16(tiled[:, hs], want, "tiled schedule")
+    assert_close_lse(auto_l[:, hs], want_l, atol=1e-2)
+    # a small grid of the same kind stays on the tiled schedule
+    small = lambda schedule: attn_vq_prefill(q[:, :2], codes[:, :2], cb[:2], v[:, :2], k_exact=k[:, :2], window_size=W,
+                                             schedule=schedule)
+    assert torch.equal(small("default"), small("tiled"))
+
+
 def test_vq_prefill_pipelined_refuses_other_configurations():
     from vqtree_amd._lib import VqaError
 

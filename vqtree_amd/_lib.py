@@ -36,6 +36,8 @@ SIGNATURES = {
     "vqa_prefill_workspace_bytes": (c_size_t, [c_int] * 4),
     "vqa_prefill_bf16": (c_int, [_P] * 10 + [c_size_t] + [c_int] * 6 + [_STRIDES, c_int, c_int, c_int, c_float, _P]),
     "vqa_prefill_f16": (c_int, [_P] * 10 + [c_size_t] + [c_int] * 6 + [_STRIDES, c_int, c_int, c_int, c_float, _P]),
+    "vqa_prefill_tiled_bf16": (c_int, [_P] * 10 + [c_size_t] + [c_int] * 6 + [_STRIDES, c_int, c_int, c_int, c_float, _P]),
+    "vqa_prefill_tiled_f16": (c_int, [_P] * 10 + [c_size_t] + [c_int] * 6 + [_STRIDES, c_int, c_int, c_int, c_float, _P]),
     "vqa_prefill_pipelined_bf16": (c_int, [_P] * 8 + [c_size_t] + [c_int] * 6 + [_STRIDES, c_int, c_int, c_float, _P]),
     "vqa_prefill_pipelined_f16": (c_int, [_P] * 8 + [c_size_t] + [c_int] * 6 + [_STRIDES, c_int, c_int, c_float, _P]),
     "vqa_prefill_f32": (c_int, [_P] * 6 + [c_int] * 6 + [_STRIDES, c_int, c_float, _P]),

@@ -16,7 +16,7 @@ namespace vqa {
 namespace count_state {
 
 constexpr int kCodesPerGroup = 16;  // codewords owned by one workgroup of count_state_add
-constexpr int kBatch = 4;           // value rows whose loads are in flight together
+constexpr int kBatch = 8;           // value rows whose loads are in flight together
 
 // grid (C / 16 code groups, B*H), D threads: thread d owns element d of the group's 16 accumulators.
 template <typename Tag, int D>

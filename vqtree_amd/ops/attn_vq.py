@@ -151,9 +151,10 @@ def attn_vq_prefill(q, k_codes, codebooks, v, *, k_exact=None, window_size=0, ca
     with q2 if given else q.  boundary(i) = max(0, floor((i - W)/128)*128) for boundary_mode "block" (the rule of
     ops/attn_vq.py:311 and of the window kernel stages), max(0, i - W) for "exact".  One softmax over all visible
     keys: the window and far parts are merged inside the kernel.  Returns out [B,H,N,D] (and base-2 lse [B,H,N]).
-    `schedule`: "default" picks the kernel (one codebook with a block boundary: the codeword-space route of
-    `vq_attn_forward`; otherwise the per-key kernel), "per_key" forces the per-key kernel, "pipelined" runs its
-    software-pipelined variant (block boundary, window a multiple of 128, no q2 / k2).
+    `schedule`: "default" picks the route (one codebook with a block boundary: the codeword-space route of
+    `vq_attn_forward`; otherwise the per-key kernel, on whichever of its two schedules the library picks for the
+    shape); "per_key" forces the per-key kernel; "tiled" / "pipelined" force the per-key kernel on that schedule
+    (pipelined: block boundary, window a multiple of 128, no q2 / k2).
     """
     from ._common import BOUNDARY, bhn_strides, check_same_16bit, last_dim_contiguous, ptr
 
@@ -197,7 +198,7 @@ def attn_vq_prefill(q, k_codes, codebooks, v, *, k_exact=None, window_size=0, ca
         *(bhn_strides(k2) if k2 is not None else dummy),
         *bhn_strides(out),
     )
-    assert schedule in ("default", "per_key", "pipelined")
+    assert schedule in ("default", "per_key", "tiled", "pipelined")
     with torch.cuda.device(q.device):
         if schedule == "pipelined":
             assert q2 is None and k2 is None and boundary_mode == "block"
@@ -206,7 +207,7 @@ def attn_vq_prefill(q, k_codes, codebooks, v, *, k_exact=None, window_size=0, ca
                 ws_bytes, B, H, N, D, M, K, strides, int(window_size), 1 if causal else 0, softmax_scale,
                 _lib.current_stream(q.device))
         else:
-            rc = getattr(lib, "vqa_prefill_" + sfx)(
+            rc = getattr(lib, ("vqa_prefill_tiled_" if schedule == "tiled" else "vqa_prefill_") + sfx)(
                 ptr(q), ptr(k_codes), ptr(codebooks), ptr(v), ptr(k_exact), ptr(q2), ptr(k2), ptr(out), ptr(lse),
                 ptr(workspace), ws_bytes, B, H, N, D, M, K, strides, int(window_size), BOUNDARY[boundary_mode],
                 1 if causal else 0, softmax_scale, _lib.current_stream(q.device))
@@ -461,7 +462,8 @@ def _remember(cache, layer_idx, ids, value_states, n_tokens, k1, key_states):
     """Record a prefill in the cache (what `update_prefill` keeps, ops/attn_vq.py:89-127): the sequence length, so
     that the next seqlen_q == 1 call is recognised as a generation step; the codeword ids and values as given; and the
     state the generation steps run on -- the count state over all keys, or, with `generation_exact_window`, the count
-    state below the far boundary of the next query plus the buffers of the exact keys above it."""
+    state below the far boundary of the next query plus the buffers of the exact keys above it.  The state itself is
+    built by the first generation step, from the tensors recorded here."""
     from .count_state import CountState, GenerationWindow
 
     if layer_idx == 0:
@@ -472,12 +474,14 @@ def _remember(cache, layer_idx, ids, value_states, n_tokens, k1, key_states):
         code_dtype = torch.uint8 if C <= 256 else torch.int16
         cache.key_codes.append(ids.to(code_dtype).unsqueeze(-1).contiguous())
         cache.value_cache.append(value_states)
-        state = CountState(B, H, C, D, value_states.device)
-        if cache.generation_exact_window:
-            state = GenerationWindow(cache.window_length, k1, key_states, value_states, ids, n_tokens, state)
-        else:
-            state.add(ids, value_states)
-        cache.decode_state.append(state)
+
+        def build():  # run by the first generation step: a prefill that is never continued does not pay for it
+            state = CountState(B, H, C, D, value_states.device)
+            if cache.generation_exact_window:
+                return GenerationWindow(cache.window_length, k1, key_states, value_states, ids, n_tokens, state)
+            return state.add(ids, value_states)
+
+        cache.decode_state.append(build)
         cache.seq_lengths.append(n_tokens)
 
 
@@ -542,6 +546,8 @@ def dispatch_attn(query_states, key_states, value_states, position_ids, cache, l
     W = cache.window_length
     t = cache.seq_lengths[layer_idx]  # position of the new token
     ids = quantize_ids(key_states, cache.codebook)
+    if callable(cache.decode_state[layer_idx]):
+        cache.decode_state[layer_idx] = cache.decode_state[layer_idx]()
     state = cache.decode_state[layer_idx]
     scale = 1 / math.sqrt(D)
     cos, sin = rope_tables(D, max(W + 2, t + 1) if cache.generation_exact_window else W + 2, rope_base,
