@@ -97,13 +97,14 @@ def _time_events(fn, steps, warmup):
         fn()
         ends[i].record()
     torch.cuda.synchronize()
-    # median: after an idle period (tensor set-up, the CPU baseline) the first ten or so calls of a compute-bound
-    # kernel run 5 - 15 % slower than the steady state (clock / power transient), hence also the long warm-ups below
+    # median: after an idle period (tensor set-up, the CPU baseline) a compute-bound kernel first slows down by ~10 %
+    # over half a dozen calls and then speeds up for another fifty (a 0.6 ms kernel: 660 -> 745 -> 555 us over 60
+    # consecutive calls; clock / power management), hence also the long warm-ups below
     ms = sorted(s.elapsed_time(e) for s, e in zip(starts, ends))
     return ms[len(ms) // 2]
 
 
-def prefill_extra(dev, steps=40, warmup=20, cpu=True):
+def prefill_extra(dev, steps=60, warmup=60, cpu=True):
     """Second half of the metric: causal VQ-attention prefill at 8k with a 1024-key exact window (not part of the
     timed decode region).  Reported as algorithmic TFLOP/s and as a fraction of the bf16 MFMA peak."""
     import torch
@@ -148,7 +149,7 @@ def prefill_extra(dev, steps=40, warmup=20, cpu=True):
     return out
 
 
-def local_rerope_extra(dev, steps=40, warmup=20, cpu=True):
+def local_rerope_extra(dev, steps=60, warmup=60, cpu=True):
     """Sliding-window ReRoPE attention at 16k (batch 2, 32 heads, window 512), the exact-window building block of the
     prefill path: useful FLOPs = 4 * D * visible pairs (keys j <= i with j >= floor(i/128)*128 - window)."""
     import torch
