@@ -8,8 +8,11 @@
  *     vqa_decode_static_bf16, works in a fixed device array of the library and says so below),
  *   - returns VQA_OK (0) or a negative vqa_status; it never throws or aborts.
  * Tensors are addressed as base + sum(index_i * stride_i) in ELEMENTS of their own type; the innermost
- * (head_dim / codebook index M) stride must be 1.  Head dims of the attention entry points: 64 and 128 (the encoder,
- * preprocessing and rotary entry points state their own limits).  The count kernel needs 64.5 KB of LDS at head dim
+ * (head_dim / codebook index M) stride must be 1.  Head dims of the attention entry points: 64 and 128; vqa_local_attn_*,
+ * vqa_rerope_full_* and vqa_vqcount_* also take 32 (the reference's kernels of these kinds accept 16, 32, 64 and 128,
+ * ops/triton_fused_attn_rerope.py:192, ops/triton_fused_vq_attn.py:198-199; a caller with head dim 16 zero-pads its
+ * operands to 32, which leaves the scores unchanged, and drops the padded output columns -- the Python layer does).
+ * The encoder, preprocessing and rotary entry points state their own limits.  The count kernel needs 64.5 KB of LDS at head dim
  * 128 and raises its dynamic-LDS limit with hipFuncSetAttribute on every call; nothing else touches process state.
  *
  * Log-sum-exp values are base 2 of the scaled scores, lse2 = log2(sum_j exp(s_ij * sm_scale)), the convention of

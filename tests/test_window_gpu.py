@@ -55,7 +55,8 @@ def test_reference_selfcheck_shapes(mode, N):
 @pytest.mark.parametrize("mode", ["strict", "loose", "rerope"])
 @pytest.mark.parametrize("B,H,N,D,W", [(2, 3, 384, 128, 128), (1, 2, 130, 128, 128), (1, 2, 257, 64, 128),
                                         (1, 1, 511, 128, 256), (2, 2, 1000, 128, 384), (1, 2, 64, 64, 128),
-                                        (1, 2, 700, 128, 1024), (1, 1, 1, 128, 128)])
+                                        (1, 2, 700, 128, 1024), (1, 1, 1, 128, 128), (2, 2, 777, 32, 128),
+                                        (1, 3, 300, 32, 256), (1, 2, 500, 16, 128)])
 def test_window_modes(mode, B, H, N, D, W):
     _say(f"window {mode} B{B} H{H} N{N} D{D} W{W}")
     q, k, v, q2, k2 = (_randn(B, H, N, D, seed=10 + s) for s in range(5))
@@ -108,7 +109,8 @@ def test_window_mask_is_exact():
 
 # ------------------------------------------------------------------ full ReRoPE
 @pytest.mark.parametrize("causal", [True, False])
-@pytest.mark.parametrize("N,D,W", [(2048, 64, 512), (700, 128, 128), (300, 128, 512), (130, 64, 64)])
+@pytest.mark.parametrize("N,D,W", [(2048, 64, 512), (700, 128, 128), (300, 128, 512), (130, 64, 64), (1100, 32, 256),
+                                   (257, 32, 64), (600, 16, 128)])
 def test_rerope_full(causal, N, D, W):
     """Includes the reference self-check shape Z=1,H=16->2,N=2048,D=64,W=512 fp16 sm_scale 0.5
     (ops/triton_fused_attn_rerope.py:253-268; it checks the non-causal call)."""
@@ -217,7 +219,8 @@ def _count_route_case(N, W, C, D, H=2, B=1, dtype=torch.float16, seed=60):
     return q1, q2, k1, k, k_hat, ids, cb, v, cnt.to(dtype), v_vq, vi
 
 
-@pytest.mark.parametrize("N,W,C,D", [(511, 256, 128, 64), (1024, 256, 256, 128), (900, 128, 512, 128)])
+@pytest.mark.parametrize("N,W,C,D", [(511, 256, 128, 64), (1024, 256, 256, 128), (900, 128, 512, 128),
+                                     (1000, 128, 256, 32), (700, 128, 128, 16)])
 def test_vq_attn_forward_reference_route(N, W, C, D):
     """vq_attn_forward on inputs built by the sort-based preprocessing, against the naive per-key oracle (includes
     the reference's own check shape: LEN=511, W=256, fp16, 2 heads of dim 64, ops/attn_vq.py:534-556)."""

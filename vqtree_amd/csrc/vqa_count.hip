@@ -218,6 +218,7 @@ int vqcount(const void* q2, const void* k_vq, const void* k_vq_cnt, const void* 
     const int zero_tiles = merge_into ? 0 : ((first < N ? first : N) + kBM - 1) / kBM;
     if (p.n_far_tiles + zero_tiles == 0) return VQA_OK;
     const dim3 grid(p.n_far_tiles + zero_tiles, B * H);
+    if (D == 32) return launch_count<Tag, 32>(p, grid, stream);
     if (D == 64) return launch_count<Tag, 64>(p, grid, stream);
     if (D == 128) return launch_count<Tag, 128>(p, grid, stream);
     return VQA_ERR_UNSUPPORTED_HEAD_DIM;

@@ -446,7 +446,7 @@ inline int validate(const Params& p, int B, int D) {
     if (B <= 0 || p.H <= 0 || p.N <= 0) return VQA_ERR_BAD_SHAPE;
     if ((int64_t)B * p.H > 65535) return VQA_ERR_BAD_ARGUMENT;
     if (p.window < 0 || !(p.scale_log2e > 0.f)) return VQA_ERR_BAD_ARGUMENT;
-    if (D != 64 && D != 128) return VQA_ERR_UNSUPPORTED_HEAD_DIM;
+    if (D != 32 && D != 64 && D != 128) return VQA_ERR_UNSUPPORTED_HEAD_DIM;
     if (!view_ok(p.qa) || !view_ok(p.qb) || !view_ok(p.ka) || !view_ok(p.kb) || !view_ok(p.kc) || !view_ok(p.v))
         return (p.qa.p && p.qb.p && p.ka.p && p.kb.p && p.kc.p && p.v.p) ? VQA_ERR_MISALIGNED : VQA_ERR_NULL_POINTER;
     if (!row_stride_ok(p.qa.sn) || !row_stride_ok(p.qb.sn) || !row_stride_ok(p.ka.sn) || !row_stride_ok(p.kb.sn) ||
@@ -457,10 +457,24 @@ inline int validate(const Params& p, int B, int D) {
     return VQA_OK;
 }
 
+// head dim 32: the window modes and the full ReRoPE mode (the reference's kernels of these kinds accept it,
+// ops/triton_fused_attn_rerope.py:192, ops/triton_fused_vq_attn.py:198-199); the additive-code prefill does not
+template <typename Tag>
+int dispatch_mode_d32(const Params& p, int B, int mode, hipStream_t stream) {
+    switch (mode) {
+        case kLocalStrict: return launch<Tag, 32, kLocalStrict>(p, B, stream);
+        case kLocalLoose: return launch<Tag, 32, kLocalLoose>(p, B, stream);
+        case kLocalRerope: return launch<Tag, 32, kLocalRerope>(p, B, stream);
+        case kFullRerope: return launch<Tag, 32, kFullRerope>(p, B, stream);
+        default: return VQA_ERR_UNSUPPORTED_HEAD_DIM;
+    }
+}
+
 template <typename Tag>
 int run(Params p, int B, int D, int mode, hipStream_t stream) {
     const int rc = validate(p, B, D);
     if (rc != VQA_OK) return rc;
+    if (D == 32) return dispatch_mode_d32<Tag>(p, B, mode, stream);
     if (D == 64) return dispatch_mode<Tag, 64>(p, B, mode, stream);
     if (D == 128) return dispatch_mode<Tag, 128>(p, B, mode, stream);
     return VQA_ERR_UNSUPPORTED_HEAD_DIM;

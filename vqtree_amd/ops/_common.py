@@ -44,9 +44,16 @@ def local_attention_bhnd(q1, q2, k1, k2, v, window_size, mode, softmax_scale, re
     _lib.require_gpu(q1, q2, k1, k2, v)
     B, H, N, D = q1.shape
     assert k1.shape == (B, H, N, D) and v.shape == (B, H, N, D), "seqlen_q == seqlen_k prefill only"
-    assert D in (64, 128), "head dimensions 64 and 128 are supported"
-    sfx = check_same_16bit(q1, q2, k1, k2, v)
+    assert D in (16, 32, 64, 128), "head dimensions 16, 32, 64 and 128 are supported"
     softmax_scale = softmax_scale or 1.0 / math.sqrt(D)
+    if D == 16:
+        # The kernels start at head dim 32 (one 32-row block of the output tile): zero-padded operands give the same
+        # scores, and the padded output columns are dropped.
+        pad = lambda x: None if x is None else torch.nn.functional.pad(x, (0, 16))
+        out, lse = local_attention_bhnd(pad(q1), pad(q2), pad(k1), pad(k2), pad(v), window_size, mode, softmax_scale,
+                                        return_lse, out_bnhd, full_causal)
+        return out[..., :16], lse
+    sfx = check_same_16bit(q1, q2, k1, k2, v)
     if out_bnhd:
         out = torch.empty((B, N, H, D), dtype=q1.dtype, device=q1.device).transpose(1, 2)
     else:

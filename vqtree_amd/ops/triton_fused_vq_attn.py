@@ -51,6 +51,10 @@ def vq_count_forward(q2, k_vq, k_vq_cnt, v_vq, vi, window_size, softmax_scale=No
     q2, k_vq, k_vq_cnt, v_vq, vi = last_dim_contiguous(q2, k_vq, k_vq_cnt, v_vq, vi)
     B, H, N, D = q2.shape
     softmax_scale = softmax_scale or 1.0 / math.sqrt(D)
+    if D == 16:  # see vq_attn_forward
+        pad = lambda x: torch.nn.functional.pad(x, (0, 16))
+        o2, l2 = vq_count_forward(pad(q2), pad(k_vq), k_vq_cnt, pad(v_vq), vi, window_size, softmax_scale)
+        return o2[..., :16], l2
     o2 = torch.empty((B, H, N, D), dtype=q2.dtype, device=q2.device)
     l2 = torch.empty((B, H, N), dtype=torch.float32, device=q2.device)
     _count_call(q2, k_vq, k_vq_cnt, v_vq, vi, window_size, softmax_scale, o2, l2, merge=False)
@@ -70,6 +74,11 @@ def vq_attn_forward(q1, q2, k1, k_vq, k_vq_cnt, k3, v, v_vq, vi, window_size, so
     q1, q2, k1, k_vq, k_vq_cnt, k3, v, v_vq, vi = last_dim_contiguous(q1, q2, k1, k_vq, k_vq_cnt, k3, v, v_vq, vi)
     B, H, N, D = q1.shape
     softmax_scale = softmax_scale or 1.0 / math.sqrt(D)
+    if D == 16:  # the kernels start at head dim 32: zero-padded operands, padded output columns dropped
+        pad = lambda x: torch.nn.functional.pad(x, (0, 16))
+        res = vq_attn_forward(pad(q1), pad(q2), pad(k1), pad(k_vq), k_vq_cnt, pad(k3), pad(v), pad(v_vq), vi,
+                              window_size, softmax_scale, return_lse)
+        return (res[0][..., :16], res[1]) if return_lse else res[..., :16]
     o1, l1 = local_attention_bhnd(q1, q2, k1, k3, v, window_size, LOCAL_REROPE, softmax_scale, True)
     # far context, merged into (o1, l1) by the count kernel's epilogue
     _count_call(q2, k_vq, k_vq_cnt, v_vq, vi, window_size, softmax_scale, o1, l1, merge=True)
