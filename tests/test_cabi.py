@@ -97,6 +97,36 @@ def test_row_strides_beyond_the_32_bit_lane_offsets_are_rejected(lib):
     assert rc == -7
 
 
+def test_count_state_and_schedule_entry_points_reject_bad_arguments_before_any_launch(lib):
+    six = _lib.strides_array(*([128] * 6))
+    add = lib.vqa_count_state_add_bf16
+    assert add(None, 16, 16, 16, 1, 1, 8, 128, 512, six, None) == -1        # ids missing
+    assert add(16, 16, 16, 16, 1, 1, 8, 48, 512, six, None) == -3          # head dim
+    assert add(16, 16, 16, 16, 0, 1, 8, 128, 512, six, None) == -2         # batch
+    assert add(16, 16, 16, 16, 1, 1, 0, 128, 512, six, None) == 0          # nothing to add: no launch, ok
+    dec = lib.vqa_count_decode_bf16
+    assert dec(16, 16, 16, 16, None, None, 1, 1, 512, 128, six, 1.0, None) == -1   # out missing
+    assert dec(16, 16, 16, 16, 16, None, 1, 1, 8193, 128, six, 1.0, None) == -2    # more codewords than the state holds
+    assert dec(16, 16, 16, 16, 16, None, 1, 1, 512, 96, six, 1.0, None) == -3
+    assert dec(16, 24, 16, 16, 16, None, 1, 1, 512, 128, six, 1.0, None) == -5     # codebook not 16-byte aligned
+    # the pipelined schedule is refused where it does not apply: window not a multiple of 128 / exact boundary rule
+    s23 = _lib.strides_array(*([128] * 23))
+    rc = lib.vqa_prefill_pipelined_bf16(16, 16, 16, 16, 16, 16, None, 256, 1 << 30, 1, 1, 256, 128, 4, 256, s23, 100, 1,
+                                        1.0, None)
+    assert rc == -7
+    # the tiled entry point validates like vqa_prefill_*: unsupported head dim, too small a workspace
+    rc = lib.vqa_prefill_tiled_bf16(16, 16, 16, 16, None, None, None, 16, None, 256, 1 << 30, 1, 1, 8, 96, 4, 256, s23,
+                                    0, 0, 1, 1.0, None)
+    assert rc == -3
+    rc = lib.vqa_prefill_tiled_bf16(16, 16, 16, 16, None, None, None, 16, None, 256, 8, 1, 1, 8, 128, 4, 256, s23, 0, 0,
+                                    1, 1.0, None)
+    assert rc == -6
+    # integer-count entry points share the count kernel's checks
+    s17 = _lib.strides_array(*([128] * 17))
+    assert lib.vqa_vqcount_fwd_icnt_bf16(16, 16, None, 16, 16, 16, None, 1, 1, 512, 128, 128, s17, 128, 1.0, None) == -1
+    assert lib.vqa_vqcount_merge_icnt_bf16(16, 16, 16, 16, 16, 16, None, 1, 1, 512, 128, 128, s17, 128, 1.0, None) == -1
+
+
 def test_static_scratch_decode_refuses_oversized_problem_on_the_host(lib):
     strides = _lib.strides_array(*([0] * 12))
     rc = lib.vqa_decode_static_bf16(16, 16, 16, 16, 16, None, 16, 32, 1 << 20, 128, 4, 256, strides, 1.0, 64, None)
