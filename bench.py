@@ -128,7 +128,11 @@ def prefill_extra(dev, steps=60, warmup=60, cpu=True):
         "tflops": round(tf, 1),
         "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
-                     "duration_covers": "whole call: key reconstruction kernel + fused window/far attention kernel"},
+                     "duration_covers": "whole call: key reconstruction kernel + fused window/far attention kernel",
+                     # attention kernel 369.7 MB fetched + 67.1 MB written, reconstruction 67.1 MB fetched + 67.1 written
+                     "traffic": 369_738_000 + 67_109_000 + 67_080_000 + 67_109_000,
+                     "traffic_source": "profiles/window_kernel_vq_prefill_c3_h32_n8192_w1024.md (rocprofv3 --pmc "
+                                       "FETCH_SIZE, then WRITE_SIZE; not measured by this run)"},
     }
     if cpu:
         # the oracle on one of the H independent heads (same inputs), rate extrapolated over heads
@@ -177,7 +181,10 @@ def local_rerope_extra(dev, steps=60, warmup=60, cpu=True):
         "tflops": round(tf, 1),
         "mfma_frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
         "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4), "duration_covers": "the one window kernel"},
+                     "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4), "duration_covers": "the one window kernel",
+                     "traffic": 2_176_082_000 + 270_157_000,
+                     "traffic_source": "profiles/window_kernel_local_rerope_c4_b2_h32_n16384_w512.md (rocprofv3 --pmc "
+                                       "FETCH_SIZE, then WRITE_SIZE; not measured by this run)"},
     }
     if cpu:
         import oracle
