@@ -74,6 +74,28 @@ def test_window_modes(mode, B, H, N, D, W):
         assert_close_lse(lse, want_lse)
 
 
+def test_full_window_causal_attention_at_a_large_shape():
+    """A window that covers the sequence is plain causal attention; at 64 heads x 4096 tokens the library runs it on
+    the pipelined schedule.  Strict and loose windows are then the same function: checked against each other, against
+    a window one short of the sequence (tiled kernel, the first row pair differs by nothing: i - j <= N - 1 always
+    holds) and, on two heads, against the oracle."""
+    _say("full-window causal H64 N4096")
+    B, H, N, D = 1, 64, 4096, 128
+    g = torch.Generator(device="cuda").manual_seed(41)
+    q, k, v = (torch.randn(B, N, H, D, generator=g, device="cuda").to(torch.bfloat16) for _ in range(3))
+    strict = triton_fused_local_attn.flash_attn_func(q, k, v, N)
+    loose, lse = triton_fused_local_attn2.flash_attn_func(q, k, v, N, return_lse=True)
+    tiled = triton_fused_local_attn.flash_attn_func(q, k, v, N - 1)  # window < N: the tiled kernel, same visible set
+    torch.cuda.synchronize()
+    assert torch.equal(strict, loose)
+    assert (strict.float() - tiled.float()).abs().max() <= 2e-2
+    hs = [3, 60]
+    bhnd = lambda x: x[:, :, hs].transpose(1, 2).cpu()
+    want, want_lse = oracle.local_attn(bhnd(q), bhnd(k), bhnd(v), N, "strict", None)
+    assert_close_16(strict[:, :, hs].transpose(1, 2), want, "full-window causal")
+    assert_close_lse(lse[:, hs], want_lse, atol=1e-2)
+
+
 def test_loose_matches_dense_ref_impl_on_device():
     q, k, v = (_bnhd(_randn(1, 2, 640, 64, seed=20 + s, std=0.5, dtype=torch.float16)).cuda() for s in range(3))
     out = triton_fused_local_attn2.flash_attn_func(q, k, v, 256, 0.5)

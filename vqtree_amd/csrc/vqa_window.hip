@@ -485,6 +485,13 @@ inline View make_view(const void* ptr, const int64_t* s) {
 }
 
 // strides: 6 tensors x (b, h, n): q1, q2, k1, k2, v, out
+// the software-pipelined kernel for the long-prefill configuration (vqa_prefill_pipe.hip)
+bool prefill_pipe_applies(int window, int boundary_is_block, bool has_exact, bool has_second_pair);
+template <typename Tag>
+int prefill_pipe_run(const View& q, const View& ka, const View& kc, const View& v, uint16_t* out, int64_t o_sb,
+                     int64_t o_sh, int64_t o_sn, float* lse, int B, int H, int N, int D, int window, int causal,
+                     bool all_far, float scale_log2e, hipStream_t stream);
+
 template <typename Tag>
 int local_attn(const void* q1, const void* q2, const void* k1, const void* k2, const void* v, void* out, float* lse,
                int B, int H, int N, int D, const int64_t* strides, int window, int mode, int causal, float sm_scale,
@@ -508,6 +515,16 @@ int local_attn(const void* q1, const void* q2, const void* k1, const void* k2, c
     p.boundary = kBoundaryBlock;
     p.has_b = 1;
     p.scale_log2e = sm_scale * kLog2e;
+    // A window that covers the whole sequence is plain causal attention: where the pipelined schedule is the faster
+    // one (same rule as in prefill() below) it runs that, every key tile an exact one.
+    if ((mode == kLocalStrict || mode == kLocalLoose) && window >= N && D == 128 && N >= 4096 &&
+        (int64_t)(((N + 255) / 256 + 1) / 2) * B * H >= 512) {
+        const int rc = validate(p, B, D);
+        if (rc != VQA_OK) return rc;
+        const int cover = (N + kTile - 1) / kTile * kTile;  // a multiple of 128 that is >= N
+        return prefill_pipe_run<Tag>(p.qa, p.ka, p.ka, p.v, p.out, p.o_sb, p.o_sh, p.o_sn, p.lse, B, H, N, D, cover, 1,
+                                     false, p.scale_log2e, stream);
+    }
     return run<Tag>(p, B, D, mode, stream);
 }
 
@@ -560,13 +577,6 @@ __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict_
         *reinterpret_cast<u32x4_t*>(kc + ((int64_t)bh * N + j0 + k) * D + col * 8) = o;
     }
 }
-
-// the software-pipelined kernel for the long-prefill configuration (vqa_prefill_pipe.hip)
-bool prefill_pipe_applies(int window, int boundary_is_block, bool has_exact, bool has_second_pair);
-template <typename Tag>
-int prefill_pipe_run(const View& q, const View& ka, const View& kc, const View& v, uint16_t* out, int64_t o_sb,
-                     int64_t o_sh, int64_t o_sn, float* lse, int B, int H, int N, int D, int window, int causal,
-                     bool all_far, float scale_log2e, hipStream_t stream);
 
 inline size_t prefill_workspace_bytes(int B, int H, int N, int D) {
     return ((size_t)B * H * N * D * 2 + 255) / 256 * 256;
