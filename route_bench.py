@@ -54,14 +54,32 @@ def run(batch=1, heads=32, tokens=8192, head_dim=128, window=1024, codes=512, de
         "count_state_build_us": _time(lambda: CountState(B, H, C, D, device).add(ids, v)),
         "dispatch_attn_whole_us": _time(lambda: A.dispatch_attn(q, k, v, pos, A.VectorQuantizedReRoPECache(W, cb))),
     }
-    # the same attention through the fused per-key kernel (needs uint8 codes: at most 256 codewords)
     cb256 = cb[:, :256].contiguous()
+    # the same attention through the fused per-key kernel (needs uint8 codes: at most 256 codewords)
     ids256 = Q.quantize_ids(k, cb256).to(torch.uint8).unsqueeze(-1)
     out["fused_per_key_256_codewords_us"] = _time(
         lambda: A.attn_vq_prefill(q1, ids256, cb256.unsqueeze(1), v, k_exact=k1, window_size=W, q2=q2, k2=k,
                                   schedule="per_key"))
     out["attn_vq_prefill_default_256_codewords_us"] = _time(  # M = 1: dispatched to the codeword-space route
         lambda: A.attn_vq_prefill(q1, ids256, cb256.unsqueeze(1), v, k_exact=k1, window_size=W, q2=q2, k2=k))
+    # one generation step after that prefill, on the cache's count state (O(C D) per step): all keys through their
+    # codewords, and with the exact window and strip of a prefill row; next to it the same attention streamed over the
+    # N one-byte codes and V rows (O(N D) per step; needs <= 256 codewords)
+    one = lambda: torch.randn(B, H, 1, D, generator=g, device=device).bfloat16()
+    qs, ks, vs = one(), one(), one()
+    for name, exact in (("generation_step_all_coded_us", False), ("generation_step_exact_window_us", True)):
+        cache = A.VectorQuantizedReRoPECache(W, cb, generation_exact_window=exact)
+        A.dispatch_attn(q, k, v, pos, cache)
+        step = [N]
+
+        def gen():
+            A.dispatch_attn(qs, ks, vs, torch.full((B, 1), step[0], device=device), cache)
+            step[0] += 1
+
+        out[name] = _time(gen, steps=20, warmup=3)  # the first call also builds the state
+    codes_u8 = Q.quantize_ids(k, cb256).to(torch.uint8).unsqueeze(-1)
+    out["generation_step_streaming_256_codewords_us"] = _time(
+        lambda: A.attn_vq_decode(qs, codes_u8, cb256.unsqueeze(1), v))
     # the four-codebook prefill benchmark workload under the two schedules of the fused kernel
     from vqtree_amd.synthetic import prefill_c3
 
