@@ -88,6 +88,17 @@ def run(batch=1, heads=32, tokens=8192, head_dim=128, window=1024, codes=512, de
         out[f"attn_vq_prefill_4x256_{schedule}_us"] = _time(
             lambda: A.attn_vq_prefill(c.q, c.codes, c.codebooks, c.v, k_exact=c.k_exact, window_size=c.window,
                                       softmax_scale=c.softmax_scale, schedule=schedule))
+    # full-context ReRoPE attention (`attention`, ops/triton_fused_attn_rerope.py:185-233) at the window benchmark's
+    # shape: batch 2, 32 heads, 16384 tokens, window 512 -- O(N^2): 4 D N (N + 1) / 2 per (batch, head) = 4 398 GFLOP
+    from vqtree_amd.ops.triton_fused_attn_rerope import attention
+
+    del q, k, v, q1, k1, q2, c
+    torch.cuda.empty_cache()
+    Bf, Nf, Wf = 2, 16384, 512
+    f1, f2, fk1, fk2, fv = (torch.randn(Bf, H, Nf, D, generator=g, device=device).bfloat16() for _ in range(5))
+    us = _time(lambda: attention(f1, f2, fk1, fk2, fv, True, 1 / D ** 0.5, Wf), steps=6, warmup=3)
+    out["rerope_full_b2_n16384_w512_us"] = us
+    out["rerope_full_b2_n16384_w512_tflops"] = round(4 * D * (Nf * (Nf + 1) / 2) * Bf * H / us / 1e6, 1)
     return out
 
 
