@@ -15,11 +15,17 @@
 namespace vqa {
 namespace count_state {
 
-constexpr int kCodesPerGroup = 16;  // codewords owned by one workgroup of count_state_add
+// Codewords owned by one workgroup of count_state_add.  A workgroup scans all T ids whatever it owns, so many keys
+// want many small groups (more workgroups in flight to hide the latency of the scan and of the row loads: 8192 keys,
+// 512 codewords, 32 heads take 251 us with 16 codewords per group and 195 us with 4), while the single key of a
+// generation step wants few, large groups (the launch is all fixed cost).
+constexpr int kCodesManyKeys = 4;
+constexpr int kCodesFewKeys = 32;
+constexpr int kManyKeys = 1024;
 constexpr int kBatch = 8;           // value rows whose loads are in flight together
 
-// grid (C / 16 code groups, B*H), D threads: thread d owns element d of the group's 16 accumulators.
-template <typename Tag, int D>
+// grid (C / kCodesPerGroup groups, B*H), D threads: thread d owns element d of the group's accumulators.
+template <typename Tag, int D, int kCodesPerGroup>
 __global__ __launch_bounds__(D) void add_kernel(const int64_t* __restrict__ ids, const uint16_t* __restrict__ v,
                                                 int32_t* __restrict__ cnt, float* __restrict__ vsum, int H, int T, int C,
                                                 int64_t i_sb, int64_t i_sh, int64_t i_st, int64_t v_sb, int64_t v_sh,
@@ -184,14 +190,17 @@ int add(const int64_t* ids, const void* v, int32_t* cnt, float* vsum, int B, int
     if (!ids || !v || !cnt || !vsum || !st) return VQA_ERR_NULL_POINTER;
     if (T == 0) return VQA_OK;
     if ((int64_t)B * H > 65535) return VQA_ERR_BAD_SHAPE;
-    const dim3 grid((C + kCodesPerGroup - 1) / kCodesPerGroup, B * H);
     const uint16_t* vp = static_cast<const uint16_t*>(v);
-    if (D == 64)
-        hipLaunchKernelGGL((add_kernel<Tag, 64>), grid, dim3(64), 0, stream, ids, vp, cnt, vsum, H, T, C, st[0], st[1],
-                           st[2], st[3], st[4], st[5]);
-    else
-        hipLaunchKernelGGL((add_kernel<Tag, 128>), grid, dim3(128), 0, stream, ids, vp, cnt, vsum, H, T, C, st[0], st[1],
-                           st[2], st[3], st[4], st[5]);
+    auto launch = [&](auto kernel, int codes_per_group, int threads) {
+        const dim3 grid((C + codes_per_group - 1) / codes_per_group, B * H);
+        hipLaunchKernelGGL(kernel, grid, dim3(threads), 0, stream, ids, vp, cnt, vsum, H, T, C, st[0], st[1], st[2],
+                           st[3], st[4], st[5]);
+    };
+    const bool many = T >= kManyKeys;
+    if (D == 64 && many) launch(add_kernel<Tag, 64, kCodesManyKeys>, kCodesManyKeys, 64);
+    if (D == 64 && !many) launch(add_kernel<Tag, 64, kCodesFewKeys>, kCodesFewKeys, 64);
+    if (D == 128 && many) launch(add_kernel<Tag, 128, kCodesManyKeys>, kCodesManyKeys, 128);
+    if (D == 128 && !many) launch(add_kernel<Tag, 128, kCodesFewKeys>, kCodesFewKeys, 128);
     return launch_status();
 }
 
