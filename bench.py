@@ -311,7 +311,11 @@ def main():
                           "frac": c5["attention_hbm_frac"],
                           "duration_covers": "HIP events around the attention calls of all 32 layers (clamped query, "
                                              "lookup table, streaming kernel, merge), per decode step, launches "
-                                             "queued ahead of the GPU"}
+                                             "queued ahead of the GPU",
+                          # streaming kernel 2 187.4 MB per layer (fetch + write counters), table and merge kernels 9.8 MB
+                          "traffic": 32 * (2_187_400_000 + 9_800_000),
+                          "traffic_source": "profiles/decode_harness_c5_b4_n65536.md (rocprofv3 --pmc FETCH_SIZE, then "
+                                            "WRITE_SIZE; not measured by this run)"}
         result["c5"] = c5
     torch.cuda.empty_cache()
     if not args.no_prefill:
