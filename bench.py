@@ -294,8 +294,9 @@ def main():
             "traffic_source": DECODE_MAIN_KERNEL_TRAFFIC["source"],
             "kernel": "vqa::decode::main_kernel<bf16,128,4>",
             "duration_us": round(kern_ms * 1e3, 1),
-            "duration_covers": "HIP events around the whole call (lookup-table + streaming + merge kernels); the "
-                               "streaming kernel is >98% of it",
+            "duration_covers": "HIP events around the whole call (lookup-table kernel + streaming kernel, which with "
+                               "one split per (batch, head) stores the result itself); the streaming kernel is 99% "
+                               "of it",
         },
     }
     if not args.no_cpu_baseline:

@@ -126,7 +126,8 @@ __global__ __launch_bounds__(kThreads, 3) void main_kernel(const uint8_t* __rest
                                                            float* __restrict__ part_o, float* __restrict__ part_ml,
                                                            int H, int N, int S, int keys_per_split, Strides st,
                                                            const int* __restrict__ n_keys_dev, int slot_stride,
-                                                           int slot_off) {
+                                                           int slot_off, uint16_t* __restrict__ out_direct,
+                                                           float* __restrict__ lse_direct) {
     constexpr int LPR = D / 8;
     constexpr int G = kWave / LPR;
     constexpr int R = kBatch / G;
@@ -278,6 +279,13 @@ __global__ __launch_bounds__(kThreads, 3) void main_kernel(const uint8_t* __rest
             for (int gg = 0; gg < G; ++gg) t += s_red[w][gg][tid];
             o += wgt * t;
             l += wgt * s_l[w];
+        }
+        if (out_direct != nullptr) {
+            // a single split whose state is the result: normalise and store, no merge launch behind this kernel
+            const int b = bh / H, h = bh % H;
+            out_direct[b * st.o_b + h * st.o_h + tid] = Elem<Tag>::to_bits(l > 0.f ? o / l : 0.f);
+            if (tid == 0 && lse_direct != nullptr) lse_direct[bh] = l > 0.f ? m_all + fast_log2(l) : -INFINITY;
+            return;
         }
         // partial states of one (batch, head) are contiguous: slot_stride of them, this launch's from slot_off on
         const int64_t slot = (int64_t)bh * slot_stride + slot_off + split;
@@ -511,10 +519,11 @@ inline int default_splits(int B, int H, int N) {
     // Measured on the streaming kernel (batch x heads from 8 to 512, 32k - 64k keys): a call is fastest with about a
     // thousand workgroups, each streaming at least 4096 keys -- more, shorter splits pay the per-workgroup prologue
     // (table copy, first loads) and a longer merge, fewer leave compute units idle.  With very few (batch, head) units
-    // shorter splits are accepted to get workgroups onto every CU at all.
+    // shorter splits are accepted to get workgroups onto every CU at all.  From 512 units on a single split per unit
+    // already keeps two workgroups on every CU, runs as fast as two splits, and needs no merge launch.
     const int64_t bh = (int64_t)B * H;
     if (bh <= 0 || N <= 0) return 1;
-    int64_t s = (1024 + bh - 1) / bh;
+    int64_t s = bh >= 512 ? 1 : (1024 + bh - 1) / bh;  // 512 units: one split each fills the chip, and needs no merge
     const int64_t min_keys = bh >= 16 ? 4096 : 1024;
     const int64_t max_s = (N + min_keys - 1) / min_keys;
     if (s > max_s) s = max_s;
@@ -526,9 +535,9 @@ inline int default_splits(int B, int H, int N) {
 template <typename Tag, int D, int M>
 int launch_main(const uint8_t* codes, const uint16_t* v, const float* lut, float* po, float* pml, int B, int H, int N,
                 int S, int kps, const Strides& st, const int* n_keys_dev, int slot_stride, int slot_off,
-                hipStream_t stream) {
+                hipStream_t stream, uint16_t* out_direct = nullptr, float* lse_direct = nullptr) {
     hipLaunchKernelGGL((main_kernel<Tag, D, M>), dim3(S, B * H), dim3(kThreads), 0, stream, codes, v, lut, po, pml, H,
-                       N, S, kps, st, n_keys_dev, slot_stride, slot_off);
+                       N, S, kps, st, n_keys_dev, slot_stride, slot_off, out_direct, lse_direct);
     return launch_status();
 }
 
@@ -554,14 +563,17 @@ int run_d(const void* q, const uint8_t* codes, const void* codebooks, const void
     // keys per split: a multiple of the workgroup's 256-key stride so only the last split is ragged
     int kps = (N + S - 1) / S;
     kps = (kps + kThreads - 1) / kThreads * kThreads;
+    // with a single split the streaming kernel's state is the result: it stores the output itself, no merge launch
+    uint16_t* direct = S == 1 ? static_cast<uint16_t*>(out) : nullptr;
+    float* direct_lse = S == 1 ? lse : nullptr;
     switch (M) {
-        case 1: rc = launch_main<Tag, D, 1>(codes, v16, lut, po, pml, B, H, N, S, kps, st, n_keys_dev, S, 0, stream); break;
-        case 2: rc = launch_main<Tag, D, 2>(codes, v16, lut, po, pml, B, H, N, S, kps, st, n_keys_dev, S, 0, stream); break;
-        case 4: rc = launch_main<Tag, D, 4>(codes, v16, lut, po, pml, B, H, N, S, kps, st, n_keys_dev, S, 0, stream); break;
-        case 8: rc = launch_main<Tag, D, 8>(codes, v16, lut, po, pml, B, H, N, S, kps, st, n_keys_dev, S, 0, stream); break;
+        case 1: rc = launch_main<Tag, D, 1>(codes, v16, lut, po, pml, B, H, N, S, kps, st, n_keys_dev, S, 0, stream, direct, direct_lse); break;
+        case 2: rc = launch_main<Tag, D, 2>(codes, v16, lut, po, pml, B, H, N, S, kps, st, n_keys_dev, S, 0, stream, direct, direct_lse); break;
+        case 4: rc = launch_main<Tag, D, 4>(codes, v16, lut, po, pml, B, H, N, S, kps, st, n_keys_dev, S, 0, stream, direct, direct_lse); break;
+        case 8: rc = launch_main<Tag, D, 8>(codes, v16, lut, po, pml, B, H, N, S, kps, st, n_keys_dev, S, 0, stream, direct, direct_lse); break;
         default: return VQA_ERR_UNSUPPORTED_CODEBOOK;
     }
-    if (rc != VQA_OK) return rc;
+    if (rc != VQA_OK || S == 1) return rc;
     hipLaunchKernelGGL((merge_kernel<Tag, D>), dim3(B * H), dim3(D), 0, stream, po, pml,
                        static_cast<uint16_t*>(out), lse, H, S, st);
     return launch_status();

@@ -172,7 +172,7 @@ def attn_vq_prefill(q, k_codes, codebooks, v, *, k_exact=None, window_size=0, ca
             and (q2 is None) == (k2 is None) and window_size % BLOCK_SIZE == 0 and N > window_size + BLOCK_SIZE):
         # One codebook: the far context is a softmax over the K codewords weighted by per-code key counts -- cost
         # O(N * K) instead of O(N^2) -- which is the reference's own formulation (ops/triton_fused_vq_attn.py:22-70).
-        # The per-key kernel below only wins its place from M = 2 on (profiles/prefill_far_path_choice.md).
+        # The per-key kernel below only wins its place from M = 2 on: 384 us against 641 us at 8192 tokens, 256 codewords.
         from .triton_fused_vq_attn import vq_attn_forward
 
         ids = k_codes[..., 0].to(torch.int64)
