@@ -24,13 +24,15 @@ def _row_reference(q_row, keys, values, scale):
     return p @ values.float()
 
 
-def test_vq_prefill_benchmark_size_sampled_rows_and_prefix():
-    print("fullsize: VQ prefill batch 1, 32 heads, 8192 tokens, window 1024", flush=True)
+@pytest.mark.parametrize("schedule", ["default", "tiled"])
+def test_vq_prefill_benchmark_size_sampled_rows_and_prefix(schedule):
+    """At this size the default call runs the pipelined schedule; "tiled" forces the other kernel."""
+    print(f"fullsize: VQ prefill batch 1, 32 heads, 8192 tokens, window 1024, schedule {schedule}", flush=True)
     case = prefill_c3("cuda")
     B, H, N, D = case.q.shape
     W = case.window
     out = attn_vq_prefill(case.q, case.codes, case.codebooks, case.v, k_exact=case.k_exact, window_size=W,
-                          softmax_scale=case.softmax_scale)
+                          softmax_scale=case.softmax_scale, schedule=schedule)
     torch.cuda.synchronize()
     bnd = oracle.far_boundary(N, W, "block")
     rows = [0, 1, 127, 128, W + 127, W + 128, W + 129, 2047, 4096, 5000, N - 129, N - 1]
@@ -45,7 +47,8 @@ def test_vq_prefill_benchmark_size_sampled_rows_and_prefix():
     # prefix property: the first 4096 tokens alone give the same rows
     half = N // 2
     out_half = attn_vq_prefill(case.q[:, :, :half], case.codes[:, :, :half], case.codebooks, case.v[:, :, :half],
-                               k_exact=case.k_exact[:, :, :half], window_size=W, softmax_scale=case.softmax_scale)
+                               k_exact=case.k_exact[:, :, :half], window_size=W, softmax_scale=case.softmax_scale,
+                               schedule=schedule)
     torch.cuda.synchronize()
     diff = (out_half.float() - out[:, :, :half].float()).abs().max().item()
     assert diff <= 2e-2, diff
