@@ -49,7 +49,7 @@ __global__ __launch_bounds__(256) void k(unsigned* out, int iters, long long* cl
         const int row = 4 * half + (sl >> 2);
         for (int i = 0; i < 32; ++i) {
             const int f = i / 2, db = f % 4, j = f / 4, hi = i % 2;
-            const int chunk = (4 * db + 2 * dsub + ((sl & 3) >> 1)) ^ (2 * (row % 8));
+            const int chunk = (4 * db + 2 * dsub + ((sl & 3) >> 1)) ^ (4 * (row % 4));
             addr[i] = base + (j * 16 + row + 8 * hi) * 256 + chunk * 16 + ((sl & 1) << 3);
         }
     }

@@ -51,10 +51,14 @@ struct Geom {
     static __device__ __forceinline__ int swz_k(int row) {
         return (int)(((unsigned)row / (unsigned)kRowsPerBankCycle) % (unsigned)kChunksPerRow);
     }
-    // chunk-index XOR of a V tile row: 8 consecutive rows x 4 consecutive chunks are read together
-    // (ds_read_b64_tr_b16); even values only, so the two 8-byte halves of a chunk stay together
+    // chunk-index XOR of a V tile row.  One ds_read_b64_tr_b16 reads 8 consecutive rows x 4 consecutive chunks (64
+    // bytes per row), its two 32-lane halves 4 rows each; the rows of a half must land in different 64-byte bank
+    // groups or they are served one after the other (measured: XOR 2*(row % 8), which maps rows 2k and 2k+1 to the
+    // same group, costs 4 LDS cycles and 2 conflict cycles per instruction; this one 2 and 0).  Multiples of 4 only:
+    // the 4 chunks of a read stay together.
     static __device__ __forceinline__ int swz_v(int row) {
-        return (int)(2u * (((unsigned)row / (unsigned)kRowsPerBankCycle) % (unsigned)(kChunksPerRow / 2)));
+        constexpr unsigned kGroups = kChunksPerRow / 4 > 0 ? kChunksPerRow / 4 : 1;  // 64-byte groups per row
+        return (int)(4u * (((unsigned)row / (unsigned)kRowsPerBankCycle) % kGroups));
     }
 };
 
