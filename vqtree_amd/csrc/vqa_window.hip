@@ -177,11 +177,12 @@ __global__ __launch_bounds__(kThreads, 2) void window_kernel(Params p) {
 
     // The workgroup walks a flat list of STEPS: step = one (key tile, operand pair) score product.  A key tile that
     // needs a single pair is one step; a tile on the window edge or the far-context boundary is one step per pair it
-    // touches, the products being merged per element.  The list runs over the key tiles of the first query tile,
-    // in the order given below, then over those of the second query tile (paired launch), so the loads of every step -- the
-    // first of a query tile included -- are requested one step ahead, and the K buffers alternate per step, the
+    // touches, the products being merged per element.  The list runs over the key tiles of the first query tile, in
+    // the order given below, then over those of the second query tile (paired launch), so the loads of every step --
+    // the first of a query tile included -- are requested one step ahead, and the K buffers alternate per step, the
     // V buffers per key tile.  Within a tile the pair scored last in the previous tile goes first, which keeps the
     // number of changes of the query operand per query tile at its minimum.
+    //
     // Order of the key tiles of one query tile.  Modes that see the whole prefix walk up from key 0: the workgroups
     // of one head start together and so read the same K / V tiles at about the same time, sharing them through
     // the L2.  Sliding-window modes walk their window in a rotated order, key tile index modulo the number of
