@@ -88,39 +88,27 @@ template <>
 struct Mai<bf16_tag> {
     // s += a . b   (a: VGPRs, b: AccVGPRs, s: VGPRs)
     static __device__ __forceinline__ void score(f32x16_t& s, u32x4_t a, u32x4_t b) {
-        asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(s) : "v"(a), "a"(b));
+        asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(s) : "a"(a), "a"(b));
     }
-    static __device__ __forceinline__ void score_first(f32x16_t& s, u32x4_t a, u32x4_t b) {
-        asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(s) : "v"(a), "a"(b));
-    }
-    // the same with b in VGPRs (query fragments that come from LDS)
-    static __device__ __forceinline__ void score_vb(f32x16_t& s, u32x4_t a, u32x4_t b) {
-        asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(s) : "v"(a), "v"(b));
-    }
-    static __device__ __forceinline__ void score_first_vb(f32x16_t& s, u32x4_t a, u32x4_t b) {
-        asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(s) : "v"(a), "v"(b));
+    // s = c + a . b   (c: a second VGPR tuple, left untouched)
+    static __device__ __forceinline__ void score_first(f32x16_t& s, u32x4_t a, u32x4_t b, const f32x16_t& c) {
+        asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %3" : "=&v"(s) : "a"(a), "a"(b), "v"(c));
     }
     // o += a . b   (a, b: VGPRs, o: AccVGPRs)
     static __device__ __forceinline__ void accumulate(f32x16_t& o, u32x4_t a, u32x4_t b) {
-        asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(o) : "v"(a), "v"(b));
+        asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(o) : "a"(a), "v"(b));
     }
 };
 template <>
 struct Mai<f16_tag> {
     static __device__ __forceinline__ void score(f32x16_t& s, u32x4_t a, u32x4_t b) {
-        asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(s) : "v"(a), "a"(b));
+        asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(s) : "a"(a), "a"(b));
     }
-    static __device__ __forceinline__ void score_first(f32x16_t& s, u32x4_t a, u32x4_t b) {
-        asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(s) : "v"(a), "a"(b));
-    }
-    static __device__ __forceinline__ void score_vb(f32x16_t& s, u32x4_t a, u32x4_t b) {
-        asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(s) : "v"(a), "v"(b));
-    }
-    static __device__ __forceinline__ void score_first_vb(f32x16_t& s, u32x4_t a, u32x4_t b) {
-        asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(s) : "v"(a), "v"(b));
+    static __device__ __forceinline__ void score_first(f32x16_t& s, u32x4_t a, u32x4_t b, const f32x16_t& c) {
+        asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %3" : "=&v"(s) : "a"(a), "a"(b), "v"(c));
     }
     static __device__ __forceinline__ void accumulate(f32x16_t& o, u32x4_t a, u32x4_t b) {
-        asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(o) : "v"(a), "v"(b));
+        asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(o) : "a"(a), "v"(b));
     }
 };
 // o *= alpha for an accumulator block that lives in AccVGPRs.  The empty volatile statement makes the block a fresh
@@ -145,25 +133,81 @@ struct Scores {
 template <typename Tag, int D>
 struct Wave {
     typedef Geom<D> G;
-    QFrag<Tag, D> q[2];            // query blocks (B operands of S^T = K.Q^T)
+    QFrag<Tag, D> q[2];            // query blocks (B operands of S^T = K.Q^T), pre-multiplied by scale * log2(e)
     f32x16_t o[2][G::kDBlocks];    // O^T accumulators
-    float m[2], l[2];              // reference maximum (base 2, scaled) and partial row sum, per block
-    float m_use[2];                // m, or 0 while the row has seen nothing
+    f32x16_t negm[2];              // -m in every element: the addend of the first score MFMA of a tile
+    float m[2];                    // reference maximum (base 2, scaled; -inf while nothing was seen), per block
+    float l[2][2];                 // two partial row sums per block (even / odd keys of the lane)
     u32x4_t p[2][4];               // packed probabilities of the current tile: [block][16-key step]
-    float ex[2][2];                // exp stream: exponentials of the unit before the current one, not packed yet
-    uint32_t pk[2];                // exp stream: packed pair of the unit two back, not summed yet
+    float ex[2][2];                // exp stream: exponentials of the current unit and of the one before
 
     __device__ __forceinline__ void init() {
 #pragma unroll
         for (int qb = 0; qb < 2; ++qb) {
             m[qb] = -INFINITY;
-            l[qb] = 0.f;
-            m_use[qb] = 0.f;
+            l[qb][0] = l[qb][1] = 0.f;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) negm[qb][i] = 0.f;
 #pragma unroll
             for (int db = 0; db < G::kDBlocks; ++db)
 #pragma unroll
                 for (int i = 0; i < 16; ++i) o[qb][db][i] = 0.f;
         }
+    }
+};
+
+// q *= c (fp32 product, one rounding to the element type).  The kernels fold softmax_scale * log2(e) into the query
+// once, so that a score leaves the matrix pipe ready for exp2.
+template <typename Tag, int D>
+__device__ __forceinline__ void prescale_q(QFrag<Tag, D>& q, float c) {
+    typedef typename Elem<Tag>::vec8 vec8;
+#pragma unroll
+    for (int kk = 0; kk < Geom<D>::kKSteps; ++kk) {
+        u32x4_t x = __builtin_bit_cast(u32x4_t, q.f[kk]);
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            x[e] = Elem<Tag>::pack2(Elem<Tag>::from_bits((uint16_t)(x[e] & 0xffffu)) * c,
+                                    Elem<Tag>::from_bits((uint16_t)(x[e] >> 16)) * c);
+        // the fragments live in AccVGPRs from here on (they are only ever an MFMA operand): defined there, the
+        // register allocator keeps them there instead of copying them in front of every product
+        asm volatile("" : "+a"(x));
+        q.f[kk] = __builtin_bit_cast(vec8, x);
+    }
+}
+
+// Copy of a whole 64-row tile, global -> LDS, with the per-lane part of the addresses computed once per kernel: load i
+// of a wave (rows 16 * wave + kRowsPerInstr * i ...) takes a wave-uniform row address (scalar registers), the lane's
+// 32-bit byte offset off[i] (row inside the group, swizzled 16-byte chunk) and an LDS address in M0.  The two halves
+// of a load -- M0 write, direct-to-LDS load -- are issued separately so that the caller can put an MFMA between them
+// (a load may not follow the M0 write directly).
+template <int D, bool kIsV>
+struct TileDma {
+    typedef Geom<D> G;
+    static constexpr int kRowsPerWave = kBN / 4;
+    static constexpr int kInstr = kRowsPerWave / G::kRowsPerInstr;
+    uint32_t off[kInstr];
+    __device__ __forceinline__ void init(int wave, int lane, int64_t sn) {
+        const int lane_row = (int)((unsigned)lane / (unsigned)G::kChunksPerRow);
+        const int chunk = (int)((unsigned)lane % (unsigned)G::kChunksPerRow);
+#pragma unroll
+        for (int i = 0; i < kInstr; ++i) {
+            const int row_in_wave = i * G::kRowsPerInstr + lane_row;
+            const int row = wave * kRowsPerWave + row_in_wave;
+            const int src_chunk = chunk ^ (kIsV ? G::swz_v(row) : G::swz_k(row));
+            off[i] = (uint32_t)row_in_wave * (uint32_t)(sn * 2) + (uint32_t)src_chunk * 16u;
+        }
+    }
+    // LDS byte address of this wave's rows inside the tile at lds_tile
+    static __device__ __forceinline__ uint32_t lds_of_wave(uint32_t lds_tile, int wave) {
+        return lds_tile + (uint32_t)(wave * kRowsPerWave * G::kRowBytes);
+    }
+    template <int I>
+    static __device__ __forceinline__ void aim(uint32_t lds_wave) {
+        asm volatile("s_add_u32 m0, %0, %1" : : "s"(lds_wave), "n"(I * G::kRowsPerInstr * G::kRowBytes) : "scc");
+    }
+    template <int I>
+    __device__ __forceinline__ void fire(const char* wave_rows) const {
+        asm volatile("global_load_lds_dwordx4 %0, %1" : : "v"(off[I]), "s"(wave_rows) : "memory");
     }
 };
 
@@ -177,24 +221,62 @@ struct Pipe {
     static constexpr int kScoreSlots = 4 * KS;  // MFMAs of S^T for both query blocks
     static constexpr int kPvSlots = 8 * DB;     // MFMAs of O^T += V^T.P^T for both query blocks
     static constexpr int kUnits = 32;           // exp units per tile: one packed pair of probabilities each
-    static constexpr int kStreamSteps = kUnits + 2;
-    static constexpr int kStepsEarly = 20;      // stream steps evaluated under the score MFMAs
-    static constexpr int kMaxUnits = 32;        // v_max3 steps of the next tile's row maxima
-    static constexpr int kAhead = 3;            // fragments read ahead of their MFMA
+
+    // The VALU work of a tile is cut into single instructions ("micro-ops") and dealt out evenly over the MFMA slots:
+    // a lone wave gets four to five VALU instructions into the shadow of one MFMA, every further one idles the matrix
+    // pipe, and an empty slot is a wasted shadow.
+    //   exp stream of the CURRENT tile: 5 micro-ops per stream step, kUnits + 1 steps (see exp_micro_op); the first
+    //   kMicroScore of them run under the score MFMAs of the NEXT tile, the rest under the first kPvStream P.V MFMAs;
+    //   row maxima of the NEXT tile: kUnits v_max3 over the P.V slots from kMaxFirst on.
+    static constexpr int kMicroOps = 5 * (kUnits + 1);
+#ifdef VQA_TUNE_MICRO_SCORE
+    static constexpr int kMicroScore = VQA_TUNE_MICRO_SCORE;
+    static constexpr int kPvStream = VQA_TUNE_PV_STREAM;
+#else
+    static constexpr int kMicroScore = D == 128 ? 100 : 80;
+    static constexpr int kPvStream = D == 128 ? 22 : 11;
+#endif
+#ifdef VQA_TUNE_MAX_FIRST
+    static constexpr int kMaxFirst = VQA_TUNE_MAX_FIRST;
+#else
+    static constexpr int kMaxFirst = D == 128 ? 16 : 2;  // (>= 2: the last score MFMA must be two MFMAs old)
+#endif
+    // micro-ops finished once slot g is through (score slots first, then the P.V slots)
+    static constexpr int micro_done(int g) {
+        if (g < 0) return 0;
+        if (g < kScoreSlots) return kMicroScore * (g + 1) / kScoreSlots;
+        const int i = g - kScoreSlots;
+        if (i >= kPvStream) return kMicroOps;
+        return kMicroScore + (kMicroOps - kMicroScore) * (i + 1) / kPvStream;
+    }
+    static constexpr int max_done(int i) {  // v_max3 units finished once P.V slot i is through
+        if (i < kMaxFirst) return 0;
+        return kUnits * (i - kMaxFirst + 1) / (kPvSlots - kMaxFirst);
+    }
+    // the probabilities of 16-key step j (units 8j .. 8j+7, packed by micro-op 5 * (unit + 1) + 2) are complete, with
+    // a slot to spare, before the first P.V MFMA that reads them
+    static constexpr bool deadlines_met() {
+        for (int j = 0; j < 4; ++j)
+            if (micro_done(kScoreSlots + 2 * DB * j - 2) < 5 * (8 * j + 8) + 3) return false;
+        return true;
+    }
+    static_assert(deadlines_met(), "the exp stream is too late for the P.V products");
+    static_assert(kPvStream <= kPvSlots && kMicroScore <= kMicroOps, "schedule out of range");
 
     // per-lane LDS address of the A fragment (row block rb, k-step 0) of a swizzled 64-row tile
-    static __device__ __forceinline__ uint32_t frag_base(const char* lds_tile, int lane) {
+    // (tiles are named by their 32-bit LDS byte address)
+    static __device__ __forceinline__ uint32_t frag_base(uint32_t lds_tile, int lane) {
         const int r = lane & 31, half = lane >> 5;
-        return flash::lds_addr_of(lds_tile) + ((uint32_t)(r * G::kRowBytes) | (uint32_t)((half ^ G::swz_k(r)) << 4));
+        return lds_tile + ((uint32_t)(r * G::kRowBytes) | (uint32_t)((half ^ G::swz_k(r)) << 4));
     }
     static __device__ __forceinline__ vec8 frag(uint32_t base, int rb, int kk) {
         const uint32_t addr = (base ^ (uint32_t)((2 * kk) << 4)) + rb * 32 * G::kRowBytes;
         return *(lds_vec8_ptr)(uintptr_t)addr;
     }
-    static __device__ __forceinline__ uint32_t vfrag_base(const char* lds_v, int lane) {
+    static __device__ __forceinline__ uint32_t vfrag_base(uint32_t lds_v, int lane) {
         const int half = lane >> 5, dsub = (lane >> 4) & 1, sl = lane & 15;
         const int row = 4 * half + (sl >> 2);
-        return flash::lds_addr_of(lds_v) +
+        return lds_v +
                ((uint32_t)(row * G::kRowBytes) | (uint32_t)(((2 * dsub + ((sl & 3) >> 1)) ^ G::swz_v(row)) << 4) |
                 (uint32_t)((sl & 1) << 3));
     }
@@ -208,162 +290,207 @@ struct Pipe {
     }
 
     // The exponentials of a tile are a stream of 32 units (one packed pair of probabilities each: unit = step*8 +
-    // block*4 + e;  16-key step = kb*2 + j2;  registers j2*8 + 2e, +1 of s[block][kb]), evaluated in three stages that
-    // are one unit apart -- stream step K does   scale/subtract + exp of unit K,   pack of unit K-1,   row sum of unit
-    // K-2   -- so that no instruction consumes the result of the one right before it (a transcendental or a pack
-    // feeding the next instruction costs wait states).  kUnits + 2 stream steps finish a tile.
-    template <int K>
-    static __device__ __forceinline__ void exp_stream_step(Wave<Tag, D>& w, const Scores& sc, float scale) {
-        if constexpr (K < kUnits) {
-            constexpr int step = K / 8, qb = (K / 4) % 2, e = K % 4;
-            constexpr int kb = step / 2, j2 = step % 2, r = j2 * 8 + 2 * e;
-            w.ex[K % 2][0] = fast_exp2(__builtin_fmaf(sc.s[qb][kb][r], scale, -w.m_use[qb]));
-            w.ex[K % 2][1] = fast_exp2(__builtin_fmaf(sc.s[qb][kb][r + 1], scale, -w.m_use[qb]));
-        }
-        if constexpr (K >= 1 && K <= kUnits) {
+    // block*4 + e;  16-key step = kb*2 + j2;  registers j2*8 + 2e, +1 of s[block][kb]), evaluated in two stages one unit
+    // apart -- stream step K does   the two exp2 of unit K,   then pack and the two row-sum additions of unit K-1   --
+    // so that no instruction consumes the result of the one right before it (a transcendental feeding the next
+    // instruction costs wait states).  Micro-op X is instruction X % 5 of stream step X / 5.  The scores arrive as
+    // scale * s - m (query pre-scaled, -m added by the first score MFMA): the exponent needs no arithmetic.
+    // The row sums are plain fp32 additions of the unrounded exponentials: v_dot2 on the packed pair would be one
+    // instruction instead of two, but the dot instructions share the matrix pipe -- next to MFMAs each costs ~8 clocks
+    // of that pipe (measured: MFMA + 4 v_dot2c 69 clocks, MFMA + 4 of any other VALU instruction 39).
+    template <int X>
+    static __device__ __forceinline__ void exp_micro_op(Wave<Tag, D>& w, const Scores& sc) {
+#ifdef VQA_KO_EXP
+        return;
+#endif
+        constexpr int K = X / 5, part = X % 5;
+        if constexpr (part < 2) {
+            if constexpr (K < kUnits) {
+                constexpr int step = K / 8, qb = (K / 4) % 2, e = K % 4;
+                constexpr int kb = step / 2, j2 = step % 2, r = j2 * 8 + 2 * e;
+                w.ex[K % 2][part] = fast_exp2(sc.s[qb][kb][r + part]);
+                pin(w.ex[K % 2][part]);
+            }
+        } else if constexpr (K >= 1) {
             constexpr int U = K - 1, step = U / 8, qb = (U / 4) % 2, e = U % 4;
-            uint32_t pk = Elem<Tag>::pack2(w.ex[U % 2][0], w.ex[U % 2][1]);
-            pin(pk);
-            w.p[qb][step][e] = pk;
-            w.pk[U % 2] = pk;
-        }
-        if constexpr (K >= 2 && K <= kUnits + 1) {
-            constexpr int U = K - 2, qb = (U / 4) % 2;
-            // sum of the ROUNDED pair, as P.V uses it
-            w.l[qb] = Elem<Tag>::dot2(w.pk[U % 2], Elem<Tag>::pack2(1.f, 1.f), w.l[qb]);
-            if constexpr (U % 4 == 3) pin(w.l[qb]);
+            if constexpr (part == 2) {
+                uint32_t pk = Elem<Tag>::pack2(w.ex[U % 2][0], w.ex[U % 2][1]);
+                pin(pk);
+                w.p[qb][step][e] = pk;
+            } else {
+                w.l[qb][part - 3] += w.ex[U % 2][part - 3];
+                pin(w.l[qb][part - 3]);
+            }
         }
     }
     // max unit IDX: mx[block] = max(mx[block], two more scores of the tile in `sn`)
     template <int IDX>
     static __device__ __forceinline__ void max_unit(float (&mx)[2], const Scores& sn) {
-        constexpr int qb = IDX / 16, t = IDX % 16, kb = t / 8, r = 2 * (t % 8);
+#ifdef VQA_KO_MAX
+        return;
+#endif
+        // the two blocks alternate, so that a v_max3 never waits for the one right before it
+        constexpr int qb = IDX % 2, t = IDX / 2, kb = t / 8, r = 2 * (t % 8);
         mx[qb] = fmaxf(fmaxf(mx[qb], sn.s[qb][kb][r]), sn.s[qb][kb][r + 1]);
-        if constexpr (t % 4 == 3) pin(mx[qb]);
+        pin(mx[qb]);
     }
 
-    // Score phase.  kMma: sn = K tile (lds_k) . Q^T for both blocks.  kExp: the first kStepsEarly steps of the exp stream of `sc`.
-    template <bool kMma, bool kExp>
-    static __device__ __forceinline__ void score_phase(Wave<Tag, D>& w, Scores& sn, const char* lds_k,
-                                                       const Scores& sc, float scale, int lane) {
-        constexpr int NF = 2 * KS;  // K fragments: (k-step, key block)
-        uint32_t base = 0;
-        vec8 kf[kAhead + 1];
-        if constexpr (kMma) {
-            base = frag_base(lds_k, opaque_lane(lane));
-#pragma unroll
-            for (int f = 0; f < kAhead; ++f) kf[f] = frag(base, f % 2, f / 2);
-        }
+    // Operand fragments travel LDS -> AccVGPRs in PAIRS (two consecutive fragments of the consumption order), the
+    // second of a pair requested first: LDS returns data in order, so the wait in front of the first use of the pair
+    // covers both, one s_waitcnt per pair instead of one per fragment (every instruction of a lone wave costs issue
+    // time, also the ones that do nothing).  kPairsAhead pairs are in flight; the first ones of a phase ("head") are
+    // requested before the phase starts, under the tail of the previous one.
+#ifdef VQA_TUNE_PAIRS_AHEAD
+    static constexpr int kPairsAhead = VQA_TUNE_PAIRS_AHEAD;
+#else
+    static constexpr int kPairsAhead = 2;
+#endif
+    static constexpr int kRingPairs = kPairsAhead + 1;
+    struct Frags {
+        vec8 f[2 * kRingPairs];
+        uint32_t base;  // per-lane LDS address of fragment 0 of the tile being read
+    };
+    // K fragment f = 2 * kk + kb (k-step kk, key block kb); pair P = k-step P
+    template <int P>
+    static __device__ __forceinline__ void load_k_pair(Frags& r) {
+        constexpr int s = (P % kRingPairs) * 2;
+#ifndef VQA_KO_LDSK
+        r.f[s + 1] = frag(r.base, 1, P);
+        __builtin_amdgcn_sched_barrier(0);
+        r.f[s] = frag(r.base, 0, P);
+        __builtin_amdgcn_sched_barrier(0);
+#endif
+    }
+    static __device__ __forceinline__ void k_head(Frags& r, uint32_t lds_k, int lane) {
+        r.base = frag_base(lds_k, lane);
+        static_for<kPairsAhead>([&](auto P) { load_k_pair<decltype(P)::value>(r); });
+    }
+    // V^T fragment f = j * DB + db (16-key step j, d block db); pair P = fragments 2P, 2P + 1
+    template <int P>
+    static __device__ __forceinline__ void load_v_pair(Frags& r) {
+        constexpr int s = (P % kRingPairs) * 2;
+#ifndef VQA_KO_LDSV
+        r.f[s + 1] = vfrag(r.base, (2 * P + 1) / DB, (2 * P + 1) % DB);
+        __builtin_amdgcn_sched_barrier(0);
+        r.f[s] = vfrag(r.base, (2 * P) / DB, (2 * P) % DB);
+        __builtin_amdgcn_sched_barrier(0);
+#endif
+    }
+    static __device__ __forceinline__ void v_head(Frags& r, uint32_t lds_v, int lane) {
+        r.base = vfrag_base(lds_v, lane);
+        static_for<kPairsAhead>([&](auto P) { load_v_pair<decltype(P)::value>(r); });
+    }
+
+    // Score phase.  kMma: sn = -m + K tile . Q^T for both blocks (kf: the tile's fragment ring, head requested).  kExp: the
+    // first kMicroScore micro-ops of the exp stream of `sc`.  kVHead: ends by requesting the head of the V tile lds_v.
+    // kDma: the wave's share of two tile copies (K tile: kd / kr, V tile: vd / vr) rides along, one load per slot with
+    // the MFMA between the M0 write and the load.
+    struct TileRequest {
+        const char* rows;  // wave-uniform global address of the wave's first row of the tile
+        uint32_t lds;      // LDS byte address of that row in the destination tile
+    };
+    typedef TileDma<D, false> KDma;
+    typedef TileDma<D, true> VDma;
+    static_assert(KDma::kInstr == VDma::kInstr && 2 * KDma::kInstr <= kScoreSlots, "tile copy does not fit the slots");
+    template <bool kMma, bool kExp, bool kVHead, bool kDma>
+    static __device__ __forceinline__ void score_phase(Wave<Tag, D>& w, Scores& sn, Frags& kf, const Scores& sc,
+                                                       Frags& vf, uint32_t lds_v, int lane, const KDma& kd,
+                                                       const TileRequest& kr, const VDma& vd, const TileRequest& vr) {
+        constexpr int NI = KDma::kInstr;
+        static_assert(kMma || !kDma, "the loads ride on the MFMA slots");
         static_for<kScoreSlots>([&](auto I) {
             constexpr int i = decltype(I)::value;
             constexpr int f = i / 2, qb = i % 2, kk = f / 2, kb = f % 2;
+            if constexpr (kDma && i < NI) KDma::template aim<i>(kr.lds);
+            if constexpr (kDma && i >= NI && i < 2 * NI) VDma::template aim<i - NI>(vr.lds);
             if constexpr (kMma) {
-                if constexpr (qb == 0 && f + kAhead < NF)
-                    kf[(f + kAhead) % (kAhead + 1)] = frag(base, (f + kAhead) % 2, (f + kAhead) / 2);
-                const u32x4_t a = __builtin_bit_cast(u32x4_t, kf[f % (kAhead + 1)]);
+                if constexpr (i % 4 == 0 && kk + kPairsAhead < KS) load_k_pair<kk + kPairsAhead>(kf);
+                const u32x4_t a = __builtin_bit_cast(u32x4_t, kf.f[(kk % kRingPairs) * 2 + kb]);
                 const u32x4_t bq = __builtin_bit_cast(u32x4_t, w.q[qb].f[kk]);
+#ifndef VQA_KO_MFMA_S
                 if constexpr (kk == 0)
-                    Mai<Tag>::score_first(sn.s[qb][kb], a, bq);
+                    Mai<Tag>::score_first(sn.s[qb][kb], a, bq, w.negm[qb]);
                 else
                     Mai<Tag>::score(sn.s[qb][kb], a, bq);
+#else
+                asm volatile("" : "+v"(sn.s[qb][kb]) : "a"(a), "a"(bq));
+#endif
             }
             if constexpr (kExp) {
-                constexpr int u0 = i * kStepsEarly / kScoreSlots, u1 = (i + 1) * kStepsEarly / kScoreSlots;
-                static_for<u1 - u0>([&](auto U) { exp_stream_step<u0 + decltype(U)::value>(w, sc, scale); });
+                constexpr int x0 = micro_done(i - 1), x1 = micro_done(i);
+                static_for<x1 - x0>([&](auto X) { exp_micro_op<x0 + decltype(X)::value>(w, sc); });
             }
+            if constexpr (kDma && i < NI) kd.template fire<i>(kr.rows);
+            if constexpr (kDma && i >= NI && i < 2 * NI) vd.template fire<i - NI>(vr.rows);
+            if constexpr (kVHead && i == kScoreSlots - 3) v_head(vf, lds_v, lane);
             __builtin_amdgcn_sched_barrier(0);
         });
     }
 
-    // P.V phase.  kPv: the rest of the exp stream of `sc` under the first half of O^T += V^T.P^T, kMax: the row maxima of
-    // `sn` under the second half.
+    // P.V phase.  kPv: O^T += V^T.P^T (vf: the V tile's fragment ring, head requested) with the rest of the exp stream of
+    // `sc` under its first MFMAs, kMax: the row maxima of `sn`.
     template <bool kPv, bool kMax>
-    static __device__ __forceinline__ void pv_phase(Wave<Tag, D>& w, const char* lds_v, const Scores& sc,
-                                                    const Scores& sn, float (&mx)[2], float scale, int lane) {
-        constexpr int NF = 4 * DB;  // V^T fragments: (16-key step, d block)
-        constexpr int kHalf = kPvSlots / 2;
-        uint32_t base = 0;
-        vec8 vf[kAhead + 1];
-        if constexpr (kPv) {
-            base = vfrag_base(lds_v, opaque_lane(lane));
-#pragma unroll
-            for (int f = 0; f < kAhead; ++f) vf[f] = vfrag(base, f / DB, f % DB);
-        } else if constexpr (kMax) {
-            mfma_settle();  // the maxima follow the score MFMAs directly
-        }
+    static __device__ __forceinline__ void pv_phase(Wave<Tag, D>& w, Frags& vf, const Scores& sc, const Scores& sn,
+                                                    float (&mx)[2]) {
+        constexpr int NP = 2 * DB;  // pairs of V^T fragments
+        if constexpr (!kPv && kMax) mfma_settle();  // the maxima follow the score MFMAs directly
         static_for<kPvSlots>([&](auto I) {
             constexpr int i = decltype(I)::value;
-            constexpr int f = i / 2, qb = i % 2, j = f / DB, db = f % DB;
+            constexpr int f = i / 2, qb = i % 2, j = f / DB, db = f % DB, pr = f / 2;
             if constexpr (kPv) {
-                if constexpr (qb == 0 && f + kAhead < NF)
-                    vf[(f + kAhead) % (kAhead + 1)] = vfrag(base, (f + kAhead) / DB, (f + kAhead) % DB);
-                Mai<Tag>::accumulate(w.o[qb][db], __builtin_bit_cast(u32x4_t, vf[f % (kAhead + 1)]), w.p[qb][j]);
-                if constexpr (i < kHalf) {
-                    constexpr int rest = kStreamSteps - kStepsEarly;
-                    constexpr int u0 = kStepsEarly + i * rest / kHalf, u1 = kStepsEarly + (i + 1) * rest / kHalf;
-                    static_for<u1 - u0>([&](auto U) { exp_stream_step<u0 + decltype(U)::value>(w, sc, scale); });
-                }
+                if constexpr (i % 4 == 0 && pr + kPairsAhead < NP) load_v_pair<pr + kPairsAhead>(vf);
+#ifndef VQA_KO_MFMA_P
+                Mai<Tag>::accumulate(w.o[qb][db], __builtin_bit_cast(u32x4_t, vf.f[(pr % kRingPairs) * 2 + f % 2]),
+                                     w.p[qb][j]);
+#else
+                asm volatile("" : "+a"(w.o[qb][db]) : "a"(__builtin_bit_cast(u32x4_t, vf.f[(pr % kRingPairs) * 2 + f % 2])), "v"(w.p[qb][j]));
+#endif
+                constexpr int x0 = micro_done(kScoreSlots + i - 1), x1 = micro_done(kScoreSlots + i);
+                static_for<x1 - x0>([&](auto X) { exp_micro_op<x0 + decltype(X)::value>(w, sc); });
             }
-            if constexpr (kMax && i >= kHalf) {
-                constexpr int u0 = (i - kHalf) * kMaxUnits / kHalf, u1 = (i - kHalf + 1) * kMaxUnits / kHalf;
+            if constexpr (kMax) {
+                constexpr int u0 = i == 0 ? 0 : max_done(i - 1), u1 = max_done(i);
                 static_for<u1 - u0>([&](auto U) { max_unit<u0 + decltype(U)::value>(mx, sn); });
             }
             __builtin_amdgcn_sched_barrier(0);
         });
     }
 
-    // Moves the reference maxima of the wave's rows for the tile whose raw row maxima are in mx (lazy rule) and
-    // rescales l / O where a row moved.  Must run after the previous tile's P.V and before this tile's exp units.
-    static __device__ __forceinline__ void update_max(Wave<Tag, D>& w, const float (&mx)[2], float scale) {
+    // Moves the reference maxima of the wave's rows for the tile whose scores are in `sc` (relative to the present
+    // maxima, as the matrix pipe delivered them) and whose per-lane maxima are in mx.  Lazy rule: a row moves only when
+    // the tile exceeds its maximum by more than 2^kLazy (or is the first one it sees).  Where a row moved, l and O are
+    // rescaled, the tile's scores are shifted to the new maximum and the addend of the coming score MFMAs is renewed.
+    // Must run after the previous tile's P.V and before this tile's exp units and the next tile's score MFMAs.
+    // The usual case -- no row of the wave moves -- is two compares and a branch: a row's maximum is the larger of the
+    // values its two lanes hold, so "some row exceeds its threshold" can be read off the lanes before they are joined.
+    static __device__ __forceinline__ void update_max(Wave<Tag, D>& w, const float (&mx)[2], Scores& sc) {
+        const bool any0 = mx[0] > ((w.m[0] == -INFINITY) ? -INFINITY : kLazy);
+        const bool any1 = mx[1] > ((w.m[1] == -INFINITY) ? -INFINITY : kLazy);
+        if (__builtin_amdgcn_ballot_w64(any0 || any1) == 0) return;
+        mfma_settle();  // O was last written by the previous tile's final MFMAs
 #pragma unroll
         for (int qb = 0; qb < 2; ++qb) {
-            const float mxs = join_halves_max(mx[qb]) * scale;  // scale > 0
-            const bool need = mxs > w.m[qb] + kLazy;             // also true for the first visible key (m = -inf)
-            if (__builtin_amdgcn_ballot_w64(need) != 0) {
-                mfma_settle();  // O was last written by the previous tile's final MFMAs
-                const float m_new = need ? mxs : w.m[qb];
-                const float alpha = need ? fast_exp2(w.m[qb] - m_new) : 1.f;  // m = -inf: alpha = 0, l = O = 0 anyway
-                w.l[qb] *= alpha;
+            const float rel = join_halves_max(mx[qb]);
+            const bool first = w.m[qb] == -INFINITY;
+            const bool need = rel > (first ? -INFINITY : kLazy);
+            const float delta = need ? rel : 0.f;
+            // a first key: l = O = 0, any finite factor keeps them there (2^-rel may overflow)
+            const float alpha = (need && !first) ? fast_exp2(-delta) : (need ? 0.f : 1.f);
+            w.l[qb][0] *= alpha;
+            w.l[qb][1] *= alpha;
 #pragma unroll
-                for (int db = 0; db < DB; ++db) rescale_acc(w.o[qb][db], alpha);
-                w.m[qb] = m_new;
-            }
-            w.m_use[qb] = (w.m[qb] == -INFINITY) ? 0.f : w.m[qb];
+            for (int db = 0; db < DB; ++db) rescale_acc(w.o[qb][db], alpha);
+            const float m_old = first ? 0.f : w.m[qb];
+            if (need) w.m[qb] = m_old + delta;
+            // (-m as old value minus delta, element by element: written like this the register allocator updates the
+            // tuple in place; a freshly built tuple ends up in other registers and is copied on the hot path)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) w.negm[qb][i] -= delta;
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) sc.s[qb][kb][i] -= delta;
         }
-    }
-
-    // Extra operand pair of a tile: s2[kb] = K tile (lds_k) . Qx^T for query block qb, with the query fragments taken
-    // from registers (kFromRegs) or from this wave's swizzled copy of the other query tensor in LDS (lds_q).
-    template <bool kFromRegs>
-    static __device__ __forceinline__ void extra_scores(f32x16_t (&s2)[2], const char* lds_k, const QFrag<Tag, D>& qreg,
-                                                        const char* lds_q, int qb, int lane) {
-        lane = opaque_lane(lane);
-        const uint32_t kbase = frag_base(lds_k, lane);
-        const uint32_t qbase = frag_base(lds_q, lane);
-        static_for<KS>([&](auto KK) {
-            constexpr int kk = decltype(KK)::value;
-            // the register-held fragments are used exactly as in the score phase (AccVGPR operand), so that they keep
-            // ONE home: a second kind of use makes the compiler park them in VGPRs and copy before every MFMA
-            u32x4_t qf;
-            if constexpr (!kFromRegs) qf = __builtin_bit_cast(u32x4_t, frag(qbase, qb, kk));
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
-                const u32x4_t a = __builtin_bit_cast(u32x4_t, frag(kbase, kb, kk));
-                if constexpr (kFromRegs) {
-                    const u32x4_t bq = __builtin_bit_cast(u32x4_t, qreg.f[kk]);
-                    if constexpr (kk == 0)
-                        Mai<Tag>::score_first(s2[kb], a, bq);
-                    else
-                        Mai<Tag>::score(s2[kb], a, bq);
-                } else {
-                    if constexpr (kk == 0)
-                        Mai<Tag>::score_first_vb(s2[kb], a, qf);
-                    else
-                        Mai<Tag>::score_vb(s2[kb], a, qf);
-                }
-            }
-        });
-        mfma_settle();
     }
 
     // Normalise and store the wave's 64 output rows; lse2 = m + log2(l).  A row that saw no key stores 0 / -inf.
@@ -373,7 +500,7 @@ struct Pipe {
         mfma_settle();
 #pragma unroll
         for (int qb = 0; qb < 2; ++qb) {
-            const float l_tot = join_halves_sum(w.l[qb]);
+            const float l_tot = join_halves_sum(w.l[qb][0] + w.l[qb][1]);
             const int row = row0 + qb * 32 + n;
             if (row >= n_rows) continue;
             const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;

@@ -44,13 +44,18 @@ template <typename Tag, int D>
 __global__ __launch_bounds__(flash2::kThreads, 1) void prefill_pipe_kernel(Params p) {
     typedef Geom<D> G;
     typedef flash2::Pipe<Tag, D> Pipe;
+    typedef typename Pipe::KDma KDma;
+    typedef typename Pipe::VDma VDma;
     extern __shared__ __attribute__((aligned(1024))) char smem[];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    auto s_ka = [&](int par) { return smem + (par & 1) * G::kTileBytes; };
-    auto s_kc = [&](int par) { return smem + (2 + (par & 1)) * G::kTileBytes; };
-    auto s_v = [&](int par) { return smem + (4 + (par & 1)) * G::kTileBytes; };
+    // tiles are named by their LDS byte address
+    const uint32_t lds0 = flash::lds_addr_of(smem);
+    auto s_ka = [&](int par) { return lds0 + (uint32_t)((par & 1) * G::kTileBytes); };
+    auto s_kc = [&](int par) { return lds0 + (uint32_t)((2 + (par & 1)) * G::kTileBytes); };
+    auto s_v = [&](int par) { return lds0 + (uint32_t)((4 + (par & 1)) * G::kTileBytes); };
+    auto lds_ptr = [&](uint32_t addr) { return smem + (addr - lds0); };
 
     // every XCD (own L2) gets whole (batch, head) problems; late and early query tiles are paired per workgroup so
     // that causal work is balanced
@@ -77,15 +82,23 @@ __global__ __launch_bounds__(flash2::kThreads, 1) void prefill_pipe_kernel(Param
     const uint16_t* v_src = p.v.p + b * p.v.sb + h * p.v.sh;
     const uint16_t* q_src = p.q.p + b * p.q.sb + h * p.q.sh;
 
-    auto copy_k = [&](const char* lds_tile, const uint16_t* base, int64_t sn, int n0) __attribute__((always_inline)) {
+    // whole-tile copies that ride on the score MFMAs: per-lane offsets once per kernel (one set per row stride)
+    KDma kd_a, kd_c;
+    VDma vd;
+    kd_a.init(wave, lane, p.ka.sn);
+    kd_c.init(wave, lane, p.kc.sn);
+    vd.init(wave, lane, p.v.sn);
+    // any other tile copy (first tiles of a pass, tiles that run over the end of the sequence, the second K source of
+    // a boundary tile): issued as a block
+    auto copy_k = [&](uint32_t lds_tile, const uint16_t* base, int64_t sn, int n0) __attribute__((always_inline)) {
         flash::TileCopy<D, false> c;
         c.init(wave, flash2::opaque_lane(lane));
-        c.load(lds_tile, base, sn, n0, p.N);
+        c.load(lds_ptr(lds_tile), base, sn, n0, p.N);
     };
-    auto copy_v = [&](const char* lds_tile, int n0) __attribute__((always_inline)) {
+    auto copy_v = [&](uint32_t lds_tile, int n0) __attribute__((always_inline)) {
         flash::TileCopy<D, true> c;
         c.init(wave, flash2::opaque_lane(lane));
-        c.load(lds_tile, v_src, p.v.sn, n0, p.N);
+        c.load(lds_ptr(lds_tile), v_src, p.v.sn, n0, p.N);
     };
 
     for (int pass = 0; pass < n_pass; ++pass) {
@@ -103,6 +116,7 @@ __global__ __launch_bounds__(flash2::kThreads, 1) void prefill_pipe_kernel(Param
     // tiles [0, n_iter): keys up to the last row of the query tile (causal) or all of them
     const int hi_key = p.causal ? min(p.N, m1 + 1) : p.N;
     const int n_iter = (hi_key + kBN - 1) / kBN;
+    const int n_whole = min(n_iter, p.N / kBN);  // tiles that lie inside the sequence with all 64 rows
     // K tiles a key tile needs (workgroup-uniform) and the buffer this wave scores from
     auto needs_far = [&](int u) { return u * kBN < fb_hi; };
     auto needs_exact = [&](int u) { return u * kBN >= fb_lo; };
@@ -115,8 +129,11 @@ __global__ __launch_bounds__(flash2::kThreads, 1) void prefill_pipe_kernel(Param
     w.init();
     flash::load_q<Tag, D>(w.q[0], q_src, p.q.sn, row0, p.N, lane);
     flash::load_q<Tag, D>(w.q[1], q_src, p.q.sn, row0 + 32, p.N, lane);
+    flash2::prescale_q<Tag, D>(w.q[0], p.scale_log2e);
+    flash2::prescale_q<Tag, D>(w.q[1], p.scale_log2e);
 
     Scores s_even, s_odd;
+    typename Pipe::Frags kf, vf;
     float mx[2] = {-INFINITY, -INFINITY};
 
     // masks of tile u for this wave: causal diagonal and end of the sequence; a tile past the wave's last row (or
@@ -143,6 +160,7 @@ __global__ __launch_bounds__(flash2::kThreads, 1) void prefill_pipe_kernel(Param
         }
     };
     auto k_tile_of_wave = [&](int u, int par) { return (u * kBN < fb_w) ? s_kc(par) : s_ka(par); };
+    const typename Pipe::TileRequest no_req{nullptr, 0};
 
     // first tile: scores, masks, row maxima (nothing to overlap with yet)
     request_k(0, 0);
@@ -150,29 +168,55 @@ __global__ __launch_bounds__(flash2::kThreads, 1) void prefill_pipe_kernel(Param
     __syncthreads();
     if (n_iter > 1) request_k(1, 1);
     copy_v(s_v(0), 0);
-    Pipe::template score_phase<true, false>(w, s_even, k_tile_of_wave(0, 0), s_odd, p.scale_log2e, lane);
+    Pipe::k_head(kf, k_tile_of_wave(0, 0), lane);
+    Pipe::template score_phase<true, false, false, false>(w, s_even, kf, s_odd, vf, 0u, lane, kd_c, no_req, vd, no_req);
     mask_tile(s_even, 0);
-    Pipe::template pv_phase<false, true>(w, s_v(0), s_odd, s_even, mx, p.scale_log2e, lane);
+    Pipe::template pv_phase<false, true>(w, vf, s_odd, s_even, mx);
 
     // Iteration u finishes tile u (exponentials, P.V) and prepares tile u + 1 (scores, masks, row maxima); K(u+1) and
-    // V(u) were requested one iteration earlier and sit in the buffers of parity u + 1 and u.
-    auto iteration = [&](auto u_is_odd, int u) __attribute__((always_inline)) {
+    // V(u) were requested one iteration earlier and sit in the buffers of parity u + 1 and u.  It requests K(u+2) and
+    // V(u+1): whole tiles ride on the score MFMAs (kRide), anything else goes out as a block in front of them.
+    auto iteration = [&](auto u_is_odd, auto ride, int u) __attribute__((always_inline)) {
         constexpr int par = decltype(u_is_odd)::value ? 1 : 0;
+        constexpr bool kRide = decltype(ride)::value;
         Scores& sc = par ? s_odd : s_even;
         Scores& sn = par ? s_even : s_odd;
-        Pipe::update_max(w, mx, p.scale_log2e);
         flash::wait_tile_loads();
         __syncthreads();  // K(u+1) and V(u) are complete; every wave is done with K(u) and V(u-1)
-        if (u + 2 < n_iter) request_k(u + 2, par);
-        if (u + 1 < n_iter) copy_v(s_v(par + 1), (u + 1) * kBN);
-        Pipe::template score_phase<true, true>(w, sn, k_tile_of_wave(u + 1, par + 1), sc, p.scale_log2e, lane);
+        Pipe::k_head(kf, k_tile_of_wave(u + 1, par + 1), lane);
+        typename Pipe::TileRequest kr = no_req, vr = no_req;
+        KDma kd = kd_c;
+        if constexpr (kRide) {
+            const int n2 = (u + 2) * kBN;
+            const bool far = needs_far(u + 2);
+            const uint16_t* src = far ? kc : ka;
+            const int64_t sn_k = far ? p.kc.sn : p.ka.sn;
+            kr.rows = reinterpret_cast<const char*>(src + (int64_t)(n2 + wave * KDma::kRowsPerWave) * sn_k);
+            kr.lds = KDma::lds_of_wave(far ? s_kc(par) : s_ka(par), wave);
+#pragma unroll
+            for (int i = 0; i < KDma::kInstr; ++i) kd.off[i] = far ? kd_c.off[i] : kd_a.off[i];
+            vr.rows = reinterpret_cast<const char*>(v_src + (int64_t)(n2 - kBN + wave * VDma::kRowsPerWave) * p.v.sn);
+            vr.lds = VDma::lds_of_wave(s_v(par + 1), wave);
+            if (far && needs_exact(u + 2)) copy_k(s_ka(par), ka, p.ka.sn, n2);  // boundary tile: both sources
+        } else {
+            if (u + 2 < n_iter) request_k(u + 2, par);
+            if (u + 1 < n_iter) copy_v(s_v(par + 1), (u + 1) * kBN);
+        }
+        Pipe::update_max(w, mx, sc);
+        Pipe::template score_phase<true, true, true, kRide>(w, sn, kf, sc, vf, s_v(par), lane, kd, kr, vd, vr);
         mask_tile(sn, u + 1);
         mx[0] = mx[1] = -INFINITY;
-        Pipe::template pv_phase<true, true>(w, s_v(par), sc, sn, mx, p.scale_log2e, lane);
+        Pipe::template pv_phase<true, true>(w, vf, sc, sn, mx);
     };
-    for (int u = 0; u < n_iter; u += 2) {
-        iteration(std::false_type{}, u);
-        if (u + 1 < n_iter) iteration(std::true_type{}, u + 1);
+    // main loop: pairs of iterations whose requests are whole tiles; then the last few, which may run over the end
+    int u = 0;
+    for (; u + 3 < n_whole; u += 2) {
+        iteration(std::false_type{}, std::true_type{}, u);
+        iteration(std::true_type{}, std::true_type{}, u + 1);
+    }
+    for (; u < n_iter; u += 2) {
+        iteration(std::false_type{}, std::false_type{}, u);
+        if (u + 1 < n_iter) iteration(std::true_type{}, std::false_type{}, u + 1);
     }
 
     Pipe::store(w, p.out + b * p.o_sb + h * p.o_sh, p.o_sn, p.lse ? p.lse + (int64_t)bh * p.N : nullptr, row0, p.N,
