@@ -340,8 +340,9 @@ def test_vq_prefill_fp32_config1(B, H, N, D, M, K, causal):
                                    (16, 96, 128)])
 def test_reconstructed_keys_are_bit_exact(M, K, D, dtype):
     """The code gathers of the prefill: the workspace of vqa_prefill_* holds K_hat = sum_m codebooks[h,m,code_m]
-    (fp32 sum in codebook order, rounded once).  Called through ctypes with a workspace of the test's own and compared
-    with the oracle's reconstruction by torch.equal."""
+    (fp32 sum in codebook order, rounded once) for every key some query scores as a far key: all of them without exact
+    keys, those below the last row's far boundary (rounded up to a block of 128) with a window.  Called through ctypes
+    with a workspace of the test's own and compared with the oracle's reconstruction by torch.equal."""
     from vqtree_amd import _lib
     from vqtree_amd.synthetic import prefill_case
 
@@ -357,17 +358,22 @@ def test_reconstructed_keys_are_bit_exact(M, K, D, dtype):
     cb = case.codebooks
     strides = _lib.strides_array(*s3(case.q), case.codes.stride(0), case.codes.stride(1), cb.stride(0), cb.stride(1),
                                  cb.stride(2), *s3(case.v), *s3(case.k_exact), 0, 0, 0, 0, 0, 0, *s3(out))
-    rc = getattr(lib, "vqa_prefill_" + sfx)(case.q.data_ptr(), case.codes.data_ptr(), cb.data_ptr(), case.v.data_ptr(),
-                                            case.k_exact.data_ptr(), None, None, out.data_ptr(), None, ws.data_ptr(),
-                                            ws_bytes, B, H, N, D, M, K, strides, 128, 0, 1, case.softmax_scale,
-                                            _lib.current_stream(case.q.device))
-    _lib.check(rc)
-    torch.cuda.synchronize()
-    k_hat = ws[: B * H * N * D * 2].view(dtype).view(B, H, N, D).cpu()
     want = oracle.reconstruct_keys(case.codes, cb).to(dtype)
-    assert torch.equal(k_hat, want)
-    want_out, _ = oracle.attn_vq_prefill(case.q, case.codes, cb, case.v, k_exact=case.k_exact, window_size=128)
-    assert_close_16(out, want_out, "prefill around the reconstruction")
+    far_keys = ((N - 1 - 128) // 128 * 128 + 127) // 128 * 128  # below the far boundary of row N - 1, in blocks of 128
+    for k_exact, n_hat in ((case.k_exact, far_keys), (None, N)):
+        ws.zero_()
+        rc = getattr(lib, "vqa_prefill_" + sfx)(case.q.data_ptr(), case.codes.data_ptr(), cb.data_ptr(),
+                                                case.v.data_ptr(), k_exact.data_ptr() if k_exact is not None else None,
+                                                None, None, out.data_ptr(), None, ws.data_ptr(), ws_bytes, B, H, N, D, M,
+                                                K, strides, 128, 0, 1, case.softmax_scale,
+                                                _lib.current_stream(case.q.device))
+        _lib.check(rc)
+        torch.cuda.synchronize()
+        k_hat = ws[: B * H * N * D * 2].view(dtype).view(B, H, N, D).cpu()
+        assert torch.equal(k_hat[:, :, :n_hat], want[:, :, :n_hat])
+        assert not k_hat[:, :, n_hat:].any()  # keys no query scores as far keys are not reconstructed
+        want_out, _ = oracle.attn_vq_prefill(case.q, case.codes, cb, case.v, k_exact=k_exact, window_size=128)
+        assert_close_16(out, want_out, "prefill around the reconstruction")
 
 
 # ------------------------------------------------------------------ software-pipelined schedule of the long prefill

@@ -173,6 +173,11 @@ __global__ __launch_bounds__(flash2::kThreads, 1) void prefill_pipe_kernel(Param
     mask_tile(s_even, 0);
     Pipe::template pv_phase<false, true>(w, vf, s_odd, s_even, mx);
 
+    // Row addresses of this wave's share of the tiles the main loop requests next: K tile u + 2, V tile u + 1.
+    const int64_t kc_step = (int64_t)kBN * p.kc.sn * 2, ka_step = (int64_t)kBN * p.ka.sn * 2, v_step = (int64_t)kBN * p.v.sn * 2;
+    const char* kc_rows = reinterpret_cast<const char*>(kc + (int64_t)(2 * kBN + wave * KDma::kRowsPerWave) * p.kc.sn);
+    const char* ka_rows = reinterpret_cast<const char*>(ka + (int64_t)(2 * kBN + wave * KDma::kRowsPerWave) * p.ka.sn);
+    const char* v_rows = reinterpret_cast<const char*>(v_src + (int64_t)(kBN + wave * VDma::kRowsPerWave) * p.v.sn);
     // Iteration u finishes tile u (exponentials, P.V) and prepares tile u + 1 (scores, masks, row maxima); K(u+1) and
     // V(u) were requested one iteration earlier and sit in the buffers of parity u + 1 and u.  It requests K(u+2) and
     // V(u+1): whole tiles ride on the score MFMAs (kRide), anything else goes out as a block in front of them.
@@ -189,15 +194,14 @@ __global__ __launch_bounds__(flash2::kThreads, 1) void prefill_pipe_kernel(Param
         if constexpr (kRide) {
             const int n2 = (u + 2) * kBN;
             const bool far = needs_far(u + 2);
-            const uint16_t* src = far ? kc : ka;
-            const int64_t sn_k = far ? p.kc.sn : p.ka.sn;
-            kr.rows = reinterpret_cast<const char*>(src + (int64_t)(n2 + wave * KDma::kRowsPerWave) * sn_k);
+            kr.rows = far ? kc_rows : ka_rows;
             kr.lds = KDma::lds_of_wave(far ? s_kc(par) : s_ka(par), wave);
 #pragma unroll
             for (int i = 0; i < KDma::kInstr; ++i) kd.off[i] = far ? kd_c.off[i] : kd_a.off[i];
-            vr.rows = reinterpret_cast<const char*>(v_src + (int64_t)(n2 - kBN + wave * VDma::kRowsPerWave) * p.v.sn);
+            vr.rows = v_rows;
             vr.lds = VDma::lds_of_wave(s_v(par + 1), wave);
             if (far && needs_exact(u + 2)) copy_k(s_ka(par), ka, p.ka.sn, n2);  // boundary tile: both sources
+            kc_rows += kc_step, ka_rows += ka_step, v_rows += v_step;
         } else {
             if (u + 2 < n_iter) request_k(u + 2, par);
             if (u + 1 < n_iter) copy_v(s_v(par + 1), (u + 1) * kBN);

@@ -530,21 +530,28 @@ int local_attn(const void* q1, const void* q2, const void* k1, const void* k2, c
 }
 
 // ---------------------------------------------------------------------------------------------------------------
-// Far-context keys: kc[b,h,j,:] = sum_m codebooks[h, m, codes[b,h,j,m], :], summed in fp32, rounded once.
-// One thread per (key, 8-element chunk); the codebooks of a head (M*K*D elements) stay L2-resident.
+// Far-context keys: kc[b,h,j,:] = sum_m codebooks[h, m, codes[b,h,j,m], :], summed in fp32, rounded once, for the keys
+// j < n_keys (the keys some query scores as far keys; the attention kernels read no others from kc).
+// One thread per (key, 8-element chunk) and kKeysPerThread keys 16 rows apart; the codebooks of a head (M*K*D elements)
+// stay L2-resident.  The kernel is bound by the latency of the chain code -> codeword row, so a thread first fetches
+// the code words of all its keys (one 4- or 8-byte load per key when M is 4 or 8 and the rows are so aligned: `wide`)
+// and then has kKeysPerThread
+// independent gathers per codebook in flight.
 // ---------------------------------------------------------------------------------------------------------------
 template <typename Tag, int D>
 __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict__ codes,
                                                       const uint16_t* __restrict__ cb, uint16_t* __restrict__ kc,
-                                                      int H, int N, int M, int K, int64_t c_sb, int64_t c_sh,
-                                                      int64_t cb_sh, int64_t cb_sm, int64_t cb_sk) {
+                                                      int H, int N, int n_keys, int M, int K, int wide,
+                                                      int64_t c_sb, int64_t c_sh, int64_t cb_sh, int64_t cb_sm,
+                                                      int64_t cb_sk) {
     constexpr int CPR = D / 8;
-    constexpr int KPT = 4;  // keys per thread: their gathers are independent and overlap
+    constexpr int KPT = 8;                 // keys per thread
+    constexpr int kRows = 256 / CPR;       // keys one pass of the workgroup covers
     const int bh = blockIdx.y;
     const int b = bh / H, h = bh % H;
-    const int idx = blockIdx.x * 256 + threadIdx.x;
-    const int j0 = (idx / CPR) * KPT, col = idx % CPR;
-    if (j0 >= N) return;
+    const int col = threadIdx.x % CPR;
+    const int j0 = blockIdx.x * (kRows * KPT) + threadIdx.x / CPR;
+    if (j0 >= n_keys) return;
     const uint8_t* code = codes + b * c_sb + h * c_sh;
     const uint16_t* cbh = cb + h * cb_sh + col * 8;
     float acc[KPT][8];
@@ -552,31 +559,67 @@ __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict_
     for (int k = 0; k < KPT; ++k)
 #pragma unroll
         for (int e = 0; e < 8; ++e) acc[k][e] = 0.f;
-    for (int m = 0; m < M; ++m) {
-        u32x4_t w[KPT];
+    auto add_rows = [&](int m0, int m_count, const uint32_t (&cw)[KPT][2]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int mm = 0; mm < 8; ++mm) {
+            if (mm >= m_count) break;
+            u32x4_t w[KPT];
+#pragma unroll
+            for (int k = 0; k < KPT; ++k) {
+                const int c = min((int)((cw[k][mm / 4] >> (8 * (mm % 4))) & 0xffu), K - 1);  // a code >= K reads codeword K - 1
+                w[k] = *reinterpret_cast<const u32x4_t*>(cbh + (m0 + mm) * cb_sm + (int64_t)c * cb_sk);
+            }
+#pragma unroll
+            for (int k = 0; k < KPT; ++k)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    acc[k][2 * e] += Elem<Tag>::from_bits((uint16_t)(w[k][e] & 0xffffu));
+                    acc[k][2 * e + 1] += Elem<Tag>::from_bits((uint16_t)(w[k][e] >> 16));
+                }
+        }
+    };
+    // code words of the thread's keys, 8 codebooks at a time
+    for (int m0 = 0; m0 < M; m0 += 8) {
+        const int m_count = min(8, M - m0);
+        uint32_t cw[KPT][2];
 #pragma unroll
         for (int k = 0; k < KPT; ++k) {
-            const int j = min(j0 + k, N - 1);
-            const int c = min((int)code[(int64_t)j * M + m], K - 1);  // a code >= K reads codeword K - 1
-            w[k] = *reinterpret_cast<const u32x4_t*>(cbh + m * cb_sm + (int64_t)c * cb_sk);
-        }
-#pragma unroll
-        for (int k = 0; k < KPT; ++k)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                acc[k][2 * e] += Elem<Tag>::from_bits((uint16_t)(w[k][e] & 0xffffu));
-                acc[k][2 * e + 1] += Elem<Tag>::from_bits((uint16_t)(w[k][e] >> 16));
+            const int j = min(j0 + k * kRows, n_keys - 1);
+            const uint8_t* cj = code + (int64_t)j * M + m0;
+            if (wide && M == 4) {
+                cw[k][0] = *reinterpret_cast<const uint32_t*>(cj);
+                cw[k][1] = 0;
+            } else if (wide && M == 8) {
+                const uint2 t = *reinterpret_cast<const uint2*>(cj);
+                cw[k][0] = t.x, cw[k][1] = t.y;
+            } else {
+                cw[k][0] = cw[k][1] = 0;
+                for (int mm = 0; mm < m_count; ++mm) cw[k][mm / 4] |= (uint32_t)cj[mm] << (8 * (mm % 4));
             }
+        }
+        add_rows(m0, m_count, cw);
     }
 #pragma unroll
     for (int k = 0; k < KPT; ++k) {
-        if (j0 + k >= N) break;
+        const int j = j0 + k * kRows;
+        if (j >= n_keys) break;
         u32x4_t o;
 #pragma unroll
         for (int e = 0; e < 4; ++e)
             o[e] = (uint32_t)Elem<Tag>::to_bits(acc[k][2 * e]) | ((uint32_t)Elem<Tag>::to_bits(acc[k][2 * e + 1]) << 16);
-        *reinterpret_cast<u32x4_t*>(kc + ((int64_t)bh * N + j0 + k) * D + col * 8) = o;
+        // whole 256-byte rows leave the wave at once: the streaming store spares the read-for-ownership of the lines
+        store_stream16(kc + ((int64_t)bh * N + j) * D + col * 8, make_uint4(o[0], o[1], o[2], o[3]));
     }
+}
+
+// Keys that some query scores as far keys: j < boundary(N - 1), rounded up to the 128-key block the attention kernels'
+// tiles are aligned to.
+inline int far_key_count(int N, int window, int boundary_mode, bool has_exact) {
+    if (!has_exact) return N;
+    const int last = N - 1 - window;
+    if (last <= 0) return 0;
+    const int nf = boundary_mode == kBoundaryBlock ? last / kTile * kTile : last;
+    return min(N, (nf + kTile - 1) / kTile * kTile);
 }
 
 inline size_t prefill_workspace_bytes(int B, int H, int N, int D) {
@@ -641,16 +684,22 @@ int prefill(const void* q, const uint8_t* codes, const void* codebooks, const vo
     int rc = validate(p, B, D);
     if (rc != VQA_OK) return rc;
 
-    const int chunks = ((N + 3) / 4) * (D / 8);  // one thread per 16-byte column of 4 consecutive keys
-    const dim3 dq_grid((chunks + 255) / 256, B * H);
-    if (D == 64)
-        hipLaunchKernelGGL((dequant_kernel<Tag, 64>), dq_grid, dim3(256), 0, stream, codes,
-                           static_cast<const uint16_t*>(codebooks), kc, H, N, M, K, s_c[0], s_c[1], s_cb[0], s_cb[1],
-                           s_cb[2]);
-    else
-        hipLaunchKernelGGL((dequant_kernel<Tag, 128>), dq_grid, dim3(256), 0, stream, codes,
-                           static_cast<const uint16_t*>(codebooks), kc, H, N, M, K, s_c[0], s_c[1], s_cb[0], s_cb[1],
-                           s_cb[2]);
+    // 4- and 8-byte code loads where every row of codes starts on such a boundary
+    const int wide = ((M == 4 || M == 8) &&
+                      !(((uintptr_t)codes | (uintptr_t)s_c[0] | (uintptr_t)s_c[1]) & (uintptr_t)(M - 1))) ? 1 : 0;
+    const int n_far = far_key_count(N, window, boundary_mode, k_exact != nullptr);
+    if (n_far > 0) {
+        const int keys_per_wg = (256 / (D / 8)) * 8;
+        const dim3 dq_grid((n_far + keys_per_wg - 1) / keys_per_wg, B * H);
+        if (D == 64)
+            hipLaunchKernelGGL((dequant_kernel<Tag, 64>), dq_grid, dim3(256), 0, stream, codes,
+                               static_cast<const uint16_t*>(codebooks), kc, H, N, n_far, M, K, wide, s_c[0], s_c[1],
+                               s_cb[0], s_cb[1], s_cb[2]);
+        else
+            hipLaunchKernelGGL((dequant_kernel<Tag, 128>), dq_grid, dim3(256), 0, stream, codes,
+                               static_cast<const uint16_t*>(codebooks), kc, H, N, n_far, M, K, wide, s_c[0], s_c[1],
+                               s_cb[0], s_cb[1], s_cb[2]);
+    }
     rc = launch_status();
     if (rc != VQA_OK) return rc;
     if (pipelined)
