@@ -139,7 +139,9 @@ int vqa_rerope_full_f16(const void* q1, const void* q2, const void* k1, const vo
  *
  *   strides[0..22]: q(b,h,n) codes(b,h) codebooks(h,m,k) v(b,h,n) k_exact(b,h,n) q2(b,h,n) k2(b,h,n) out(b,h,n);
  *   code rows are packed (stride(n) = M).  M in [1,16], K <= 256, D in {64,128}.
- *   workspace: >= vqa_prefill_workspace_bytes(B,H,N,D) bytes, 256-byte aligned (holds the reconstructed keys).
+ *   workspace: >= vqa_prefill_workspace_bytes(B,H,N,D) bytes, 256-byte aligned.  On return it holds the reconstructed
+ *   keys [B,H,N,D] of every key some query scores as a quantised key: all of them when k_exact == NULL, else the keys
+ *   below boundary(N - 1), rounded up to a block of 128 (the rest of the buffer is not written).
  * ------------------------------------------------------------------------------------------------------------------ */
 #define VQA_BOUNDARY_BLOCK 0
 #define VQA_BOUNDARY_EXACT 1
@@ -163,8 +165,8 @@ int vqa_prefill_f16(const void* q, const uint8_t* codes, const void* codebooks, 
  *                under the score MFMAs of the next one; only for the reference's long-prefill configuration: no
  *                second query / key pair, the block boundary rule, `window` a multiple of 128 (or k_exact == NULL:
  *                every key quantised).
- * It takes the pipelined one where that is measurably faster on MI355X (3 - 7 %): when it applies, D == 128,
- * N >= 4096 and the launch has at least 512 workgroups (two rounds for the 256 CUs).  The two entry points below force
+ * It takes the pipelined one where it applies and N >= 2048 (measured on MI355X over batch x heads 1 - 256, head dims 64
+ * and 128, 1k - 32k tokens: 0.69 - 0.96 of the tiled kernel's time from 2048 tokens on).  The two entry points below force
  * a schedule: vqa_prefill_tiled_* has vqa_prefill_*'s signature; vqa_prefill_pipelined_* returns VQA_ERR_BAD_ARGUMENT
  * where the pipelined schedule does not apply (same strides array, the q2 / k2 slots are ignored).  Same workspace,
  * same results within the 16-bit tolerance.  Counterpart in the reference: the two launches of

@@ -400,9 +400,9 @@ def test_vq_prefill_pipelined_schedule(B, H, N, D, M, W, dtype):
 
 
 def test_vq_prefill_schedule_choice_at_a_large_shape():
-    """64 heads x 4096 tokens (512 workgroups of 256 query rows in pairs): vqa_prefill_* takes the pipelined schedule
-    here.  The default call must be bit-identical to the forced pipelined one, within tolerance of the forced tiled
-    one, and two heads are checked against the oracle (heads are independent)."""
+    """64 heads x 4096 tokens: vqa_prefill_* takes the pipelined schedule from 2048 tokens on.  The default call must
+    be bit-identical to the forced pipelined one, within tolerance of the forced tiled one, and two heads are checked
+    against the oracle (heads are independent)."""
     _say("vq prefill schedule choice H64 N4096")
     B, H, N, D, M, W = 1, 64, 4096, 128, 4, 1024
     g = torch.Generator(device="cuda").manual_seed(97)
@@ -421,9 +421,10 @@ def test_vq_prefill_schedule_choice_at_a_large_shape():
     assert_close_16(auto[:, hs], want, "auto schedule")
     assert_close_16(tiled[:, hs], want, "tiled schedule")
     assert_close_lse(auto_l[:, hs], want_l, atol=1e-2)
-    # a small grid of the same kind stays on the tiled schedule
-    small = lambda schedule: attn_vq_prefill(q[:, :2], codes[:, :2], cb[:2], v[:, :2], k_exact=k[:, :2], window_size=W,
-                                             schedule=schedule)
+    # a short sequence of the same kind stays on the tiled schedule
+    n = 1536
+    small = lambda schedule: attn_vq_prefill(q[:, :2, :n], codes[:, :2, :n], cb[:2], v[:, :2, :n], k_exact=k[:, :2, :n],
+                                             window_size=W, schedule=schedule)
     assert torch.equal(small("default"), small("tiled"))
 
 

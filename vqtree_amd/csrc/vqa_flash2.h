@@ -7,8 +7,18 @@
 // With a single wave per SIMD nothing else hides the softmax behind the matrix pipe, so the wave does it itself: the
 // scores of key tile u+1 are accumulated (S^T = K.Q^T, v_mfma_f32_32x32x16) while the exponentials of tile u are
 // evaluated, and the row maxima of tile u+1 are taken while P(u).V(u) runs.  The code is written as MFMA "slots":
-// slot i issues one MFMA (and the LDS read of a fragment a few slots ahead) followed by its share of the VALU work;
-// scheduling barriers between slots keep that interleaving.
+// slot i issues one MFMA followed by its share of everything else (VALU work, LDS fragment reads a few slots ahead,
+// tile copies); scheduling barriers between slots keep that interleaving.
+//
+// What bounds a lone wave is instruction ISSUE: it issues one instruction every 5 - 6 clocks whatever its kind (an
+// exponential every 9), an MFMA occupies the matrix pipe for 32, so about four other instructions fit in the shadow
+// of an MFMA and every further one idles the pipe.  The loop is therefore written for instruction COUNT:
+//   * the query is pre-multiplied by scale * log2(e) and the first score MFMA of a tile adds -m (a register tuple per
+//     query block as its C operand), so a score leaves the pipe ready for exp2: no per-score multiply-add;
+//   * row sums are fp32 additions, not v_dot2 (the dot instructions execute on the matrix pipe);
+//   * fragments are read from LDS in pairs with one s_waitcnt per pair, tile copies take two instructions per load
+//     and ride on the MFMA slots, per-lane addresses are computed once, the usual case of the maximum update is two
+//     compares and a branch.
 //
 // Layouts (as in vqa_flash.h): scores are transposed, a lane (n = lane % 32, half = lane / 32) holds ONE query column
 // per 32-row block, so row statistics are per-lane scalars (one v_permlane32_swap joins the halves) and the
@@ -75,18 +85,17 @@ __device__ __forceinline__ void pin(T& x) {
 }
 
 // MFMA forms with the register file chosen by hand.  The compiler's allocator does not find the split this kernel
-// needs by itself (O^T and the query fragments in AccVGPRs, everything the VALU touches in VGPRs) and spills; inline
-// assembly pins it.  The compiler inserts no hazard wait states around inline assembly: an MFMA result is read by
-// another MFMA only several MFMAs later (independent accumulation chains), and `mfma_settle()` stands wherever the
-// VALU may read a result that the last few instructions produced.  The forms that take an AccVGPR operand start with
-// two wait states of their own: when the compiler parks a query fragment in VGPRs it copies it (v_accvgpr_write)
-// right in front of the statement, and an MFMA may not read a register a VALU instruction wrote in the two cycles
-// before.
+// needs by itself (O^T, the query fragments and the K / V^T fragments in AccVGPRs, everything the VALU touches in
+// VGPRs) and spills; inline assembly pins it.  The compiler inserts no hazard wait states around inline assembly: an
+// MFMA result is read by another MFMA only several MFMAs later (independent accumulation chains), `mfma_settle()`
+// stands wherever the VALU may read a result that the last few instructions produced, and no MFMA operand is
+// written by a VALU instruction in the slot before it (the query fragments are DEFINED in AccVGPRs, see prescale_q,
+// so the compiler has no copy to place there; the probabilities are packed at least a slot ahead).
 template <typename Tag>
 struct Mai;
 template <>
 struct Mai<bf16_tag> {
-    // s += a . b   (a: VGPRs, b: AccVGPRs, s: VGPRs)
+    // s += a . b   (a, b: AccVGPRs, s: VGPRs)
     static __device__ __forceinline__ void score(f32x16_t& s, u32x4_t a, u32x4_t b) {
         asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(s) : "a"(a), "a"(b));
     }
@@ -94,7 +103,7 @@ struct Mai<bf16_tag> {
     static __device__ __forceinline__ void score_first(f32x16_t& s, u32x4_t a, u32x4_t b, const f32x16_t& c) {
         asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %3" : "=&v"(s) : "a"(a), "a"(b), "v"(c));
     }
-    // o += a . b   (a, b: VGPRs, o: AccVGPRs)
+    // o += a . b   (a: AccVGPRs, b: VGPRs, o: AccVGPRs)
     static __device__ __forceinline__ void accumulate(f32x16_t& o, u32x4_t a, u32x4_t b) {
         asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(o) : "a"(a), "v"(b));
     }
@@ -300,9 +309,6 @@ struct Pipe {
     // of that pipe (measured: MFMA + 4 v_dot2c 69 clocks, MFMA + 4 of any other VALU instruction 39).
     template <int X>
     static __device__ __forceinline__ void exp_micro_op(Wave<Tag, D>& w, const Scores& sc) {
-#ifdef VQA_KO_EXP
-        return;
-#endif
         constexpr int K = X / 5, part = X % 5;
         if constexpr (part < 2) {
             if constexpr (K < kUnits) {
@@ -326,9 +332,6 @@ struct Pipe {
     // max unit IDX: mx[block] = max(mx[block], two more scores of the tile in `sn`)
     template <int IDX>
     static __device__ __forceinline__ void max_unit(float (&mx)[2], const Scores& sn) {
-#ifdef VQA_KO_MAX
-        return;
-#endif
         // the two blocks alternate, so that a v_max3 never waits for the one right before it
         constexpr int qb = IDX % 2, t = IDX / 2, kb = t / 8, r = 2 * (t % 8);
         mx[qb] = fmaxf(fmaxf(mx[qb], sn.s[qb][kb][r]), sn.s[qb][kb][r + 1]);
@@ -354,12 +357,10 @@ struct Pipe {
     template <int P>
     static __device__ __forceinline__ void load_k_pair(Frags& r) {
         constexpr int s = (P % kRingPairs) * 2;
-#ifndef VQA_KO_LDSK
         r.f[s + 1] = frag(r.base, 1, P);
         __builtin_amdgcn_sched_barrier(0);
         r.f[s] = frag(r.base, 0, P);
         __builtin_amdgcn_sched_barrier(0);
-#endif
     }
     static __device__ __forceinline__ void k_head(Frags& r, uint32_t lds_k, int lane) {
         r.base = frag_base(lds_k, lane);
@@ -369,12 +370,10 @@ struct Pipe {
     template <int P>
     static __device__ __forceinline__ void load_v_pair(Frags& r) {
         constexpr int s = (P % kRingPairs) * 2;
-#ifndef VQA_KO_LDSV
         r.f[s + 1] = vfrag(r.base, (2 * P + 1) / DB, (2 * P + 1) % DB);
         __builtin_amdgcn_sched_barrier(0);
         r.f[s] = vfrag(r.base, (2 * P) / DB, (2 * P) % DB);
         __builtin_amdgcn_sched_barrier(0);
-#endif
     }
     static __device__ __forceinline__ void v_head(Frags& r, uint32_t lds_v, int lane) {
         r.base = vfrag_base(lds_v, lane);
@@ -407,14 +406,10 @@ struct Pipe {
                 if constexpr (i % 4 == 0 && kk + kPairsAhead < KS) load_k_pair<kk + kPairsAhead>(kf);
                 const u32x4_t a = __builtin_bit_cast(u32x4_t, kf.f[(kk % kRingPairs) * 2 + kb]);
                 const u32x4_t bq = __builtin_bit_cast(u32x4_t, w.q[qb].f[kk]);
-#ifndef VQA_KO_MFMA_S
                 if constexpr (kk == 0)
                     Mai<Tag>::score_first(sn.s[qb][kb], a, bq, w.negm[qb]);
                 else
                     Mai<Tag>::score(sn.s[qb][kb], a, bq);
-#else
-                asm volatile("" : "+v"(sn.s[qb][kb]) : "a"(a), "a"(bq));
-#endif
             }
             if constexpr (kExp) {
                 constexpr int x0 = micro_done(i - 1), x1 = micro_done(i);
@@ -439,12 +434,8 @@ struct Pipe {
             constexpr int f = i / 2, qb = i % 2, j = f / DB, db = f % DB, pr = f / 2;
             if constexpr (kPv) {
                 if constexpr (i % 4 == 0 && pr + kPairsAhead < NP) load_v_pair<pr + kPairsAhead>(vf);
-#ifndef VQA_KO_MFMA_P
                 Mai<Tag>::accumulate(w.o[qb][db], __builtin_bit_cast(u32x4_t, vf.f[(pr % kRingPairs) * 2 + f % 2]),
                                      w.p[qb][j]);
-#else
-                asm volatile("" : "+a"(w.o[qb][db]) : "a"(__builtin_bit_cast(u32x4_t, vf.f[(pr % kRingPairs) * 2 + f % 2])), "v"(w.p[qb][j]));
-#endif
                 constexpr int x0 = micro_done(kScoreSlots + i - 1), x1 = micro_done(kScoreSlots + i);
                 static_for<x1 - x0>([&](auto X) { exp_micro_op<x0 + decltype(X)::value>(w, sc); });
             }

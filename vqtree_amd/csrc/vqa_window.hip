@@ -487,6 +487,7 @@ inline View make_view(const void* ptr, const int64_t* s) {
 
 // strides: 6 tensors x (b, h, n): q1, q2, k1, k2, v, out
 // the software-pipelined kernel for the long-prefill configuration (vqa_prefill_pipe.hip)
+constexpr int kPipeMinTokens = 2048;  // shorter sequences stay on the tiled schedule
 bool prefill_pipe_applies(int window, int boundary_is_block, bool has_exact, bool has_second_pair);
 template <typename Tag>
 int prefill_pipe_run(const View& q, const View& ka, const View& kc, const View& v, uint16_t* out, int64_t o_sb,
@@ -518,8 +519,7 @@ int local_attn(const void* q1, const void* q2, const void* k1, const void* k2, c
     p.scale_log2e = sm_scale * kLog2e;
     // A window that covers the whole sequence is plain causal attention: where the pipelined schedule is the faster
     // one (same rule as in prefill() below) it runs that, every key tile an exact one.
-    if ((mode == kLocalStrict || mode == kLocalLoose) && window >= N && D == 128 && N >= 4096 &&
-        (int64_t)(((N + 255) / 256 + 1) / 2) * B * H >= 512) {
+    if ((mode == kLocalStrict || mode == kLocalLoose) && window >= N && (D == 64 || D == 128) && N >= kPipeMinTokens) {
         const int rc = validate(p, B, D);
         if (rc != VQA_OK) return rc;
         const int cover = (N + kTile - 1) / kTile * kTile;  // a multiple of 128 that is >= N
@@ -545,7 +545,7 @@ __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict_
                                                       int64_t c_sb, int64_t c_sh, int64_t cb_sh, int64_t cb_sm,
                                                       int64_t cb_sk) {
     constexpr int CPR = D / 8;
-    constexpr int KPT = 8;                 // keys per thread
+    constexpr int KPT = 4;                 // keys per thread
     constexpr int kRows = 256 / CPR;       // keys one pass of the workgroup covers
     const int bh = blockIdx.y;
     const int b = bh / H, h = bh % H;
@@ -638,15 +638,10 @@ int prefill(const void* q, const uint8_t* codes, const void* codebooks, const vo
     const bool pipe_ok = prefill_pipe_applies(window, boundary_mode == kBoundaryBlock, k_exact != nullptr,
                                               k_exact && q2 && k2);
     if (schedule == kSchedulePipelined && !pipe_ok) return VQA_ERR_BAD_ARGUMENT;
-    // Measured over batch x heads from 2 to 256 and 1.5k - 32k tokens: the pipelined schedule (256-row query tiles, one
-    // workgroup per CU) is 3 - 7 % faster once there are two rounds of workgroups for the 256 CUs and the sequences
-    // are long enough to amortise its longer prologue, at head dim 128; it is slower (up to 1.4 x) on small grids
-    // and level at head dim 64.
-    bool pipelined = schedule == kSchedulePipelined;
-    if (schedule == kScheduleAuto && pipe_ok && D == 128 && N >= 4096) {
-        const int64_t n_wg = (int64_t)(((N + 255) / 256 + 1) / 2) * B * H;
-        pipelined = n_wg >= 512;
-    }
+    // Measured over batch x heads from 1 to 256, 1k - 32k tokens, head dims 64 and 128: the pipelined schedule
+    // (256-row query tiles, one workgroup per CU) is the faster one from 2048 tokens on (0.69 - 0.96 of the tiled
+    // kernel's time, the more the longer the sequence); at 1024 tokens its longer prologue makes it level or slower.
+    const bool pipelined = schedule == kSchedulePipelined || (schedule == kScheduleAuto && pipe_ok && N >= kPipeMinTokens);
     if (B <= 0 || H <= 0 || N <= 0) return VQA_ERR_BAD_SHAPE;
     if (D != 64 && D != 128) return VQA_ERR_UNSUPPORTED_HEAD_DIM;
     if (M < 1 || M > 16 || K < 1 || K > 256) return VQA_ERR_UNSUPPORTED_CODEBOOK;
@@ -689,7 +684,7 @@ int prefill(const void* q, const uint8_t* codes, const void* codebooks, const vo
                       !(((uintptr_t)codes | (uintptr_t)s_c[0] | (uintptr_t)s_c[1]) & (uintptr_t)(M - 1))) ? 1 : 0;
     const int n_far = far_key_count(N, window, boundary_mode, k_exact != nullptr);
     if (n_far > 0) {
-        const int keys_per_wg = (256 / (D / 8)) * 8;
+        const int keys_per_wg = (256 / (D / 8)) * 4;  // kRows * KPT of dequant_kernel
         const dim3 dq_grid((n_far + keys_per_wg - 1) / keys_per_wg, B * H);
         if (D == 64)
             hipLaunchKernelGGL((dequant_kernel<Tag, 64>), dq_grid, dim3(256), 0, stream, codes,
