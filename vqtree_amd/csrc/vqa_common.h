@@ -132,4 +132,22 @@ inline bool row_stride_ok(int64_t sn) { return sn >= 0 && sn < (int64_t(1) << 24
 
 inline int launch_status() { return hipGetLastError() == hipSuccess ? VQA_OK : VQA_ERR_LAUNCH_FAILED; }
 
+// Per-device set-up (a kernel attribute raised once, the address of a file-scope device array) belongs to the device
+// that OWNS the memory a call works on, which need not be the calling thread's current device.  Returns that device
+// for a device pointer, VQA_ERR_BAD_ARGUMENT if it is not the current device (the launch that follows would run on
+// the current one), VQA_ERR_LAUNCH_FAILED if the runtime cannot tell.
+constexpr int kMaxDevices = 64;
+inline int device_of_pointer(const void* ptr, int* device) {
+    int cur = 0;
+    if (hipGetDevice(&cur) != hipSuccess || cur < 0 || cur >= kMaxDevices) return VQA_ERR_LAUNCH_FAILED;
+    hipPointerAttribute_t attr;
+    if (ptr != nullptr && hipPointerGetAttributes(&attr, ptr) == hipSuccess) {
+        if (attr.type == hipMemoryTypeDevice && attr.device != cur) return VQA_ERR_BAD_ARGUMENT;
+    } else {
+        (void)hipGetLastError();  // not a pointer the runtime knows (host code tests pass such): current device
+    }
+    *device = cur;
+    return VQA_OK;
+}
+
 }  // namespace vqa

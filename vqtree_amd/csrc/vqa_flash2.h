@@ -130,14 +130,20 @@ __device__ __forceinline__ void rescale_acc(f32x16_t& o, float alpha) {
     asm volatile("" : "+a"(o));
 }
 
-// 16 wait states: more than an 8-pass MFMA needs before the VALU may read its result
+// 16 wait states: more than an 8-pass MFMA needs before the VALU may read its result.  The values that must not be
+// read earlier are operands of the statement: a compiler-generated read may be moved across a volatile statement it
+// does not depend on (only volatile statements keep their order among themselves), so the wait is tied to the data.
 __device__ __forceinline__ void mfma_settle() { asm volatile("s_nop 15" ::: "memory"); }
+__device__ __forceinline__ void mfma_settle(f32x16_t& x) { asm volatile("s_nop 15" : "+v"(x)::"memory"); }
 
 // Scores of one key tile for the wave's two query blocks: s[qb][kb], accumulator layout of vqa_flash.h
 // (lane (n, half), register r  <->  key kb*32 + 8*(r/4) + 4*half + r%4 of query n of block qb).
 struct Scores {
     f32x16_t s[2][2];
 };
+__device__ __forceinline__ void mfma_settle(Scores& sc) {
+    asm volatile("s_nop 15" : "+v"(sc.s[0][0]), "+v"(sc.s[0][1]), "+v"(sc.s[1][0]), "+v"(sc.s[1][1])::"memory");
+}
 
 template <typename Tag, int D>
 struct Wave {
@@ -189,10 +195,10 @@ __device__ __forceinline__ void prescale_q(QFrag<Tag, D>& q, float c) {
 // 32-bit byte offset off[i] (row inside the group, swizzled 16-byte chunk) and an LDS address in M0.  The two halves
 // of a load -- M0 write, direct-to-LDS load -- are issued separately so that the caller can put an MFMA between them
 // (a load may not follow the M0 write directly).
-template <int D, bool kIsV>
+template <int D, bool kIsV, int NW = 4>
 struct TileDma {
     typedef Geom<D> G;
-    static constexpr int kRowsPerWave = kBN / 4;
+    static constexpr int kRowsPerWave = kBN / NW;  // NW waves share a tile copy
     static constexpr int kInstr = kRowsPerWave / G::kRowsPerInstr;
     uint32_t off[kInstr];
     __device__ __forceinline__ void init(int wave, int lane, int64_t sn) {
@@ -220,7 +226,7 @@ struct TileDma {
     }
 };
 
-template <typename Tag, int D>
+template <typename Tag, int D, int NW = 4>
 struct Pipe {
     typedef Geom<D> G;
     typedef typename Elem<Tag>::vec8 vec8;
@@ -388,8 +394,8 @@ struct Pipe {
         const char* rows;  // wave-uniform global address of the wave's first row of the tile
         uint32_t lds;      // LDS byte address of that row in the destination tile
     };
-    typedef TileDma<D, false> KDma;
-    typedef TileDma<D, true> VDma;
+    typedef TileDma<D, false, NW> KDma;
+    typedef TileDma<D, true, NW> VDma;
     static_assert(KDma::kInstr == VDma::kInstr && 2 * KDma::kInstr <= kScoreSlots, "tile copy does not fit the slots");
     template <bool kMma, bool kExp, bool kVHead, bool kDma>
     static __device__ __forceinline__ void score_phase(Wave<Tag, D>& w, Scores& sn, Frags& kf, const Scores& sc,
@@ -425,10 +431,10 @@ struct Pipe {
     // P.V phase.  kPv: O^T += V^T.P^T (vf: the V tile's fragment ring, head requested) with the rest of the exp stream of
     // `sc` under its first MFMAs, kMax: the row maxima of `sn`.
     template <bool kPv, bool kMax>
-    static __device__ __forceinline__ void pv_phase(Wave<Tag, D>& w, Frags& vf, const Scores& sc, const Scores& sn,
+    static __device__ __forceinline__ void pv_phase(Wave<Tag, D>& w, Frags& vf, const Scores& sc, Scores& sn,
                                                     float (&mx)[2]) {
         constexpr int NP = 2 * DB;  // pairs of V^T fragments
-        if constexpr (!kPv && kMax) mfma_settle();  // the maxima follow the score MFMAs directly
+        if constexpr (!kPv && kMax) mfma_settle(sn);  // the maxima follow the score MFMAs directly
         static_for<kPvSlots>([&](auto I) {
             constexpr int i = decltype(I)::value;
             constexpr int f = i / 2, qb = i % 2, j = f / DB, db = f % DB, pr = f / 2;
@@ -484,18 +490,49 @@ struct Pipe {
         }
     }
 
+    // Second operand pair of a tile (ReRoPE window edge): where take(qb, kb, r) holds, the score of `sn` is replaced by
+    // -m + K tile (lds_k) . q^T with the wave's CURRENT query fragments.  One accumulation chain at a time with a
+    // 16-register temporary; nothing is overlapped with it (it runs once per query tile and wave).
+    template <typename Take>
+    static __device__ __forceinline__ void second_pair(Wave<Tag, D>& w, Scores& sn, uint32_t lds_k, int lane,
+                                                       Take take) {
+        const uint32_t base = frag_base(lds_k, opaque_lane(lane));
+        static_for<4>([&](auto C) {
+            constexpr int qb = decltype(C)::value / 2, kb = decltype(C)::value % 2;
+            f32x16_t t;
+            static_for<KS>([&](auto KK) {
+                constexpr int kk = decltype(KK)::value;
+                const u32x4_t a = __builtin_bit_cast(u32x4_t, frag(base, kb, kk));
+                const u32x4_t bq = __builtin_bit_cast(u32x4_t, w.q[qb].f[kk]);
+                if constexpr (kk == 0)
+                    Mai<Tag>::score_first(t, a, bq, w.negm[qb]);
+                else
+                    Mai<Tag>::score(t, a, bq);
+            });
+            mfma_settle(t);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) sn.s[qb][kb][r] = take(qb, kb, r) ? t[r] : sn.s[qb][kb][r];
+        });
+    }
+
     // Normalise and store the wave's 64 output rows; lse2 = m + log2(l).  A row that saw no key stores 0 / -inf.
+    // In the accumulator layout a lane holds 4-element pieces of ONE row: stored directly, every instruction would
+    // touch 64 rows.  The rows go through the wave's own LDS staging area instead (kStoreBytes at lds_stage, rows
+    // padded by 8 bytes so that the 8-byte pieces of 32 rows fall into different banks) and leave as whole 256-byte
+    // rows, 16 bytes per lane.  The caller makes sure no wave still reads what lies in that LDS area.
+    static constexpr int kStoreRowBytes = G::kRowBytes + 8;
+    static constexpr int kStoreBytes = kWaveRows * kStoreRowBytes;
     static __device__ __forceinline__ void store(const Wave<Tag, D>& w, uint16_t* out_base, int64_t sn, float* lse,
-                                                 int row0, int n_rows, int lane) {
+                                                 int row0, int n_rows, int lane, char* lds_stage) {
         const int n = lane & 31, half = lane >> 5;
         mfma_settle();
 #pragma unroll
         for (int qb = 0; qb < 2; ++qb) {
+#pragma unroll
+            for (int db = 0; db < DB; ++db) asm volatile("" : "+a"(const_cast<f32x16_t&>(w.o[qb][db])));  // read after the wait
             const float l_tot = join_halves_sum(w.l[qb][0] + w.l[qb][1]);
-            const int row = row0 + qb * 32 + n;
-            if (row >= n_rows) continue;
             const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-            uint16_t* dst = out_base + (int64_t)row * sn;
+            char* dst = lds_stage + (qb * 32 + n) * kStoreRowBytes;
 #pragma unroll
             for (int db = 0; db < DB; ++db) {
 #pragma unroll
@@ -506,10 +543,24 @@ struct Pipe {
                            ((uint32_t)Elem<Tag>::to_bits(w.o[qb][db][4 * g + 1] * inv) << 16);
                     pk.y = (uint32_t)Elem<Tag>::to_bits(w.o[qb][db][4 * g + 2] * inv) |
                            ((uint32_t)Elem<Tag>::to_bits(w.o[qb][db][4 * g + 3] * inv) << 16);
-                    *reinterpret_cast<uint2*>(dst + db * 32 + 8 * g + 4 * half) = pk;
+                    *reinterpret_cast<uint2*>(dst + (db * 32 + 8 * g + 4 * half) * 2) = pk;
                 }
             }
-            if (lse != nullptr && half == 0) lse[row] = l_tot > 0.f ? w.m[qb] + fast_log2(l_tot) : -INFINITY;
+            const int row = row0 + qb * 32 + n;
+            if (lse != nullptr && half == 0 && row < n_rows)
+                lse[row] = l_tot > 0.f ? w.m[qb] + fast_log2(l_tot) : -INFINITY;
+        }
+        wave_lds_sync();
+        constexpr int kLanesPerRow = G::kRowBytes / 16, kRowsPerInstr = 64 / kLanesPerRow;
+        const int r_in = lane / kLanesPerRow, c = lane % kLanesPerRow;
+#pragma unroll
+        for (int i = 0; i < kWaveRows / kRowsPerInstr; ++i) {
+            const int r = i * kRowsPerInstr + r_in;
+            // (8-byte reads: the padded rows are only 8-byte aligned)
+            const uint2 lo = *reinterpret_cast<const uint2*>(lds_stage + r * kStoreRowBytes + c * 16);
+            const uint2 hi = *reinterpret_cast<const uint2*>(lds_stage + r * kStoreRowBytes + c * 16 + 8);
+            if (row0 + r < n_rows)
+                *reinterpret_cast<uint4*>(out_base + (int64_t)(row0 + r) * sn + c * 8) = make_uint4(lo.x, lo.y, hi.x, hi.y);
         }
     }
 };

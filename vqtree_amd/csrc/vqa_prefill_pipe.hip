@@ -1,15 +1,25 @@
-// Long-context VQ prefill on the software-pipelined core (vqa_flash2.h): causal attention whose far keys
-// (j < boundary(i)) are scored against the reconstructed keys K_hat and whose recent keys against the exact keys, both
-// with the same query tensor, boundary(i) = max(0, floor((i - W) / 128) * 128) with W a multiple of 128 -- the
-// configuration of the reference's long prefill (ops/attn_vq.py:311, window lengths are multiples of its 128 block) --
-// or every key far (no exact keys).  Everything else (a second query / key pair for the strip between boundary and
-// window, the exact boundary rule, other window lengths) stays with the general kernel in vqa_window.hip.
+// Long sequences on the software-pipelined core (vqa_flash2.h), three kinds of causal attention (Kind):
 //
-// What makes this case simple: a wave's 64 query rows lie inside one 128-row block, so they share one boundary and,
-// with 64-key tiles, every (wave, tile) block uses ONE key source.  A workgroup's two 128-row blocks differ by one
-// 128-key step, so for two tiles per query tile the workgroup brings both the exact and the reconstructed K tile and
-// each wave reads the one it needs; no per-element selection exists, masks only on the causal diagonal and at the
-// end of the sequence.  The tile schedule is plain arithmetic on (m0, W, N).
+//   kVq      VQ prefill: far keys (j < boundary(i)) are scored against the reconstructed keys K_hat, recent keys against
+//            the exact keys, both with the same query tensor, boundary(i) = max(0, floor((i - W) / 128) * 128) with W a
+//            multiple of 128 -- the configuration of the reference's long prefill (ops/attn_vq.py:311, window lengths
+//            are multiples of its 128 block) -- or every key far (no exact keys).
+//   kWindow  sliding window with one operand pair: keys j <= i with j >= i - W (strict) or j >= floor(i/128)*128 - W
+//            (the reference's block rule, ops/triton_fused_local_attn2.py), W a multiple of 128.
+//   kRerope  the block-rule window with the ReRoPE pair rule (ops/triton_fused_local_attn_rerope.py:38-78): score
+//            q1.k1 where i - j <= W, else q2.k2.
+//
+// Everything else (a second query / key pair next to quantised keys, the exact boundary rule, other window lengths)
+// stays with the general kernel in vqa_window.hip.
+//
+// What makes these cases simple: a wave's 64 query rows lie inside one 128-row block, so they share one boundary and,
+// with 64-key tiles, every (wave, tile) block uses ONE key source -- but for the one tile per wave that the ReRoPE
+// window edge crosses, which gets a second product.  A workgroup's waves differ by a few 64-key steps, so for a few
+// tiles per query tile the workgroup brings both K sources and each wave reads the one it needs; no per-element
+// selection exists elsewhere, masks only on the causal diagonal, at the lower window edge and at the end of the
+// sequence.  The tile schedule is plain arithmetic on (m0, W, N).
+#include <mutex>
+
 #include "vqa_flash2.h"
 
 namespace vqa {
@@ -19,31 +29,51 @@ using flash::Geom;
 using flash::View;
 using flash2::Scores;
 
-constexpr int kBM = flash2::kBM;
 constexpr int kBN = flash2::kBN;
-constexpr int kBlock = 128;  // granularity of the far-context boundary
+constexpr int kBlock = 128;  // granularity of the far-context boundary and of the block-rule window
+
+enum Kind : int { kVq = 0, kWindow = 1, kRerope = 2 };
 
 struct Params {
-    View q, ka, kc, v;  // ka: exact keys (unused when all_far), kc: reconstructed keys
+    View q, q2, ka, kc, v;  // ka: exact keys / first pair (unused when all_far), kc: reconstructed keys / second pair
     uint16_t* out;
     int64_t o_sb, o_sh, o_sn;
     float* lse;  // [B,H,N] contiguous, nullable
     int H, N, window;
-    int causal, all_far;
+    int causal, all_far;  // kVq
+    int strict;           // kWindow: j >= i - W instead of the block rule
     int pair_tiles;
     float scale_log2e;
 };
 
-// LDS: exact-K tiles [2] | reconstructed-K tiles [2] | V tiles [2]
-template <int D>
+// Workgroup shapes.  kVq: 4 waves = 256 query rows, one workgroup per CU (long key loops; the tile copies serve 256
+// rows).  Window kinds: 2 waves = 128 query rows and TWO workgroups per CU: a query tile meets only (W + 128) / 64 key
+// tiles, so the start of a workgroup (first tiles and queries from a cold start) and its end (output rows) are a
+// large part of its life and must overlap with another workgroup's products; 128-row tiles also waste fewer
+// (wave, tile) blocks below the window (a wave idles while the waves of the other 128-row block still have keys).
+template <int KIND>
+constexpr int waves_of() {
+    return KIND == kVq ? 4 : 2;
+}
+// LDS: first-source K tiles [2] | V tiles [2] | second-source K tiles: [2] for kVq, [1] for kRerope (two workgroups
+// must fit the 160 KB: only the first two key tiles of a query tile have a second source, the second one is brought
+// when the first has been scored), none for kWindow
+template <int KIND>
+constexpr int second_source_slots() {
+    return KIND == kVq ? 2 : (KIND == kRerope ? 1 : 0);
+}
+template <int D, int KIND>
 constexpr size_t lds_bytes() {
-    return (size_t)Geom<D>::kTileBytes * 6;
+    return (size_t)Geom<D>::kTileBytes * (4 + second_source_slots<KIND>());
 }
 
-template <typename Tag, int D>
-__global__ __launch_bounds__(flash2::kThreads, 1) void prefill_pipe_kernel(Params p) {
+template <typename Tag, int D, int KIND>
+__global__ __launch_bounds__(64 * waves_of<KIND>(), 1) void prefill_pipe_kernel(Params p) {
     typedef Geom<D> G;
-    typedef flash2::Pipe<Tag, D> Pipe;
+    constexpr int NW = waves_of<KIND>();
+    constexpr int kBM = NW * flash2::kWaveRows;  // query rows per workgroup
+    constexpr int kSlotsC = second_source_slots<KIND>();
+    typedef flash2::Pipe<Tag, D, NW> Pipe;
     typedef typename Pipe::KDma KDma;
     typedef typename Pipe::VDma VDma;
     extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -53,8 +83,8 @@ __global__ __launch_bounds__(flash2::kThreads, 1) void prefill_pipe_kernel(Param
     // tiles are named by their LDS byte address
     const uint32_t lds0 = flash::lds_addr_of(smem);
     auto s_ka = [&](int par) { return lds0 + (uint32_t)((par & 1) * G::kTileBytes); };
-    auto s_kc = [&](int par) { return lds0 + (uint32_t)((2 + (par & 1)) * G::kTileBytes); };
-    auto s_v = [&](int par) { return lds0 + (uint32_t)((4 + (par & 1)) * G::kTileBytes); };
+    auto s_v = [&](int par) { return lds0 + (uint32_t)((2 + (par & 1)) * G::kTileBytes); };
+    auto s_kc = [&](int par) { return lds0 + (uint32_t)((4 + (kSlotsC == 2 ? (par & 1) : 0)) * G::kTileBytes); };
     auto lds_ptr = [&](uint32_t addr) { return smem + (addr - lds0); };
 
     // every XCD (own L2) gets whole (batch, head) problems; late and early query tiles are paired per workgroup so
@@ -81,6 +111,7 @@ __global__ __launch_bounds__(flash2::kThreads, 1) void prefill_pipe_kernel(Param
     const uint16_t* kc = p.kc.p + b * p.kc.sb + h * p.kc.sh;
     const uint16_t* v_src = p.v.p + b * p.v.sb + h * p.v.sh;
     const uint16_t* q_src = p.q.p + b * p.q.sb + h * p.q.sh;
+    const uint16_t* q2_src = p.q2.p + b * p.q2.sb + h * p.q2.sh;
 
     // whole-tile copies that ride on the score MFMAs: per-lane offsets once per kernel (one set per row stride)
     KDma kd_a, kd_c;
@@ -91,12 +122,12 @@ __global__ __launch_bounds__(flash2::kThreads, 1) void prefill_pipe_kernel(Param
     // any other tile copy (first tiles of a pass, tiles that run over the end of the sequence, the second K source of
     // a boundary tile): issued as a block
     auto copy_k = [&](uint32_t lds_tile, const uint16_t* base, int64_t sn, int n0) __attribute__((always_inline)) {
-        flash::TileCopy<D, false> c;
+        flash::TileCopy<D, false, NW> c;
         c.init(wave, flash2::opaque_lane(lane));
         c.load(lds_ptr(lds_tile), base, sn, n0, p.N);
     };
     auto copy_v = [&](uint32_t lds_tile, int n0) __attribute__((always_inline)) {
-        flash::TileCopy<D, true> c;
+        flash::TileCopy<D, true, NW> c;
         c.init(wave, flash2::opaque_lane(lane));
         c.load(lds_ptr(lds_tile), v_src, p.v.sn, n0, p.N);
     };
@@ -108,76 +139,119 @@ __global__ __launch_bounds__(flash2::kThreads, 1) void prefill_pipe_kernel(Param
     const int row0 = m0 + wave * flash2::kWaveRows;  // this wave's 64 rows (inside one 128-row block)
     if (pass) __syncthreads();  // the previous query tile's last reads of the LDS buffers are done
 
-    // first exact key of the two 128-row blocks of the workgroup, and of this wave's block
     const int kNever = 0x7fffffff;
-    const int fb_lo = p.all_far ? kNever : max(0, m0 - p.window);
-    const int fb_hi = p.all_far ? kNever : max(0, m0 + kBlock - p.window);
-    const int fb_w = (wave < 2) ? fb_lo : fb_hi;
-    // tiles [0, n_iter): keys up to the last row of the query tile (causal) or all of them
-    const int hi_key = p.causal ? min(p.N, m1 + 1) : p.N;
+    // kVq: first exact key of the two 128-row blocks of the workgroup, and of this wave's block
+    const int fb_lo = (KIND != kVq || p.all_far) ? kNever : max(0, m0 - p.window);
+    const int fb_hi = (KIND != kVq || p.all_far) ? kNever : max(0, m0 + kBM - kBlock - p.window);
+    const int fb_w = (wave * flash2::kWaveRows < kBlock) ? fb_lo : fb_hi;
+    // kRerope: the second pair scores the keys j < i - W: whole tiles below edge_w, half of the tile at edge_w
+    const int edge_w = KIND == kRerope ? row0 - p.window : -1;
+    // window kinds: lowest visible key of the wave's rows (lo_w + row offset for the strict rule) and of the query tile
+    const int lo_w = KIND == kVq ? 0 : (p.strict ? row0 - p.window : (row0 / kBlock) * kBlock - p.window);
+    // tiles [u0, n_iter): from the query tile's lowest visible key up to its last row (causal) or all keys
+    const int u0 = KIND == kVq ? 0 : max(0, m0 - p.window) / kBN;
+    const int hi_key = (KIND != kVq || p.causal) ? min(p.N, m1 + 1) : p.N;
     const int n_iter = (hi_key + kBN - 1) / kBN;
     const int n_whole = min(n_iter, p.N / kBN);  // tiles that lie inside the sequence with all 64 rows
     // K tiles a key tile needs (workgroup-uniform) and the buffer this wave scores from
-    auto needs_far = [&](int u) { return u * kBN < fb_hi; };
-    auto needs_exact = [&](int u) { return u * kBN >= fb_lo; };
-    auto request_k = [&](int u, int par) __attribute__((always_inline)) {
-        if (needs_far(u)) copy_k(s_kc(par), kc, p.kc.sn, u * kBN);
-        if (needs_exact(u)) copy_k(s_ka(par), ka, p.ka.sn, u * kBN);
+    auto needs_c = [&](int u) {
+        if (KIND == kVq) return u * kBN < fb_hi;
+        if (KIND == kRerope) return u * kBN <= m0 + (NW - 1) * flash2::kWaveRows - p.window;  // the last wave's edge tile
+        return false;
     };
+    auto needs_a = [&](int u) { return KIND == kVq ? u * kBN >= fb_lo : true; };
+    // (a single second-source slot holds the tile being scored: the next one cannot be requested ahead, see iteration)
+    auto request_k = [&](int u, int par) __attribute__((always_inline)) {
+        if (needs_c(u) && (kSlotsC == 2 || u == u0)) copy_k(s_kc(par), kc, p.kc.sn, u * kBN);
+        if (needs_a(u)) copy_k(s_ka(par), ka, p.ka.sn, u * kBN);
+    };
+    auto wave_reads_c = [&](int u) { return KIND == kVq ? u * kBN < fb_w : (KIND == kRerope && u * kBN <= edge_w); };
+
+    // the first tiles are requested before anything else of the pass: their latency covers the query loads
+    request_k(u0, 0);
+    copy_v(s_v(0), u0 * kBN);
+    if (u0 + 1 < n_iter) request_k(u0 + 1, 1);
 
     flash2::Wave<Tag, D> w;
     w.init();
-    flash::load_q<Tag, D>(w.q[0], q_src, p.q.sn, row0, p.N, lane);
-    flash::load_q<Tag, D>(w.q[1], q_src, p.q.sn, row0 + 32, p.N, lane);
-    flash2::prescale_q<Tag, D>(w.q[0], p.scale_log2e);
-    flash2::prescale_q<Tag, D>(w.q[1], p.scale_log2e);
+    {
+        // kRerope: a wave that meets second-pair keys starts with the second query and changes over at its edge tile
+        const uint16_t* src = (KIND == kRerope && edge_w >= 0) ? q2_src : q_src;
+        const int64_t sn_q = (KIND == kRerope && edge_w >= 0) ? p.q2.sn : p.q.sn;
+        flash::load_q<Tag, D>(w.q[0], src, sn_q, row0, p.N, lane);
+        flash::load_q<Tag, D>(w.q[1], src, sn_q, row0 + 32, p.N, lane);
+        flash2::prescale_q<Tag, D>(w.q[0], p.scale_log2e);
+        flash2::prescale_q<Tag, D>(w.q[1], p.scale_log2e);
+    }
 
     Scores s_even, s_odd;
     typename Pipe::Frags kf, vf;
     float mx[2] = {-INFINITY, -INFINITY};
 
-    // masks of tile u for this wave: causal diagonal and end of the sequence; a tile past the wave's last row (or
-    // past the last tile) ends up fully masked
+    // masks of tile u for this wave: causal diagonal, lower window edge and end of the sequence; a tile past the
+    // wave's last row (or past the last tile) ends up fully masked
     auto mask_tile = [&](Scores& sn, int u) __attribute__((always_inline)) {
         const int n0 = u * kBN;
-        const bool whole = (n0 + kBN <= p.N) && (!p.causal || n0 + kBN - 1 <= row0) && u < n_iter;
+        const bool causal = KIND != kVq || p.causal;
+        const int lo_last = lo_w + ((KIND == kWindow && p.strict) ? flash2::kWaveRows - 1 : 0);  // of the wave's last row
+        const bool whole = (n0 + kBN <= p.N) && (!causal || n0 + kBN - 1 <= row0) && u < n_iter &&
+                           (KIND == kVq || n0 >= lo_last);
         if (whole) return;  // (wave-uniform)
-        flash2::mfma_settle();  // the scores below were produced by the last MFMAs
+        flash2::mfma_settle(sn);  // the scores below were produced by the last MFMAs
         const int lane_o = flash2::opaque_lane(lane);  // keeps the predicates inside this branch
         const int half = lane_o >> 5;
         const int j_hi = u < n_iter ? p.N : 0;  // no such tile: nothing visible
 #pragma unroll
         for (int qb = 0; qb < 2; ++qb) {
             const int i = row0 + qb * 32 + (lane_o & 31);
-            const int lim = p.causal ? min(j_hi, i + 1) : j_hi;  // keys j < lim are visible
+            const int lim = causal ? min(j_hi, i + 1) : j_hi;  // keys lo <= j < lim are visible
+            const int lo = KIND == kVq ? 0 : lo_w + ((KIND == kWindow && p.strict) ? i - row0 : 0);
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int j = n0 + kb * 32 + flash::key_of_reg(r, half);
-                    sn.s[qb][kb][r] = j < lim ? sn.s[qb][kb][r] : -INFINITY;
+                    const bool vis = KIND == kVq ? j < lim : (j < lim && j >= lo);
+                    sn.s[qb][kb][r] = vis ? sn.s[qb][kb][r] : -INFINITY;
                 }
         }
     };
-    auto k_tile_of_wave = [&](int u, int par) { return (u * kBN < fb_w) ? s_kc(par) : s_ka(par); };
+    // after the scores of tile u: masks, and at the wave's ReRoPE edge tile the change-over to the first pair (the
+    // scores so far are q2.k2; keys with i - j <= W take q1.k1, and q1 serves every later tile)
+    auto finish_scores = [&](Scores& sn, int u, int par) __attribute__((always_inline)) {
+        mask_tile(sn, u);
+        if constexpr (KIND == kRerope) {
+            if (u * kBN == edge_w) {  // (wave-uniform; every key of this tile is visible to every row of the wave)
+                flash::load_q<Tag, D>(w.q[0], q_src, p.q.sn, row0, p.N, lane);
+                flash::load_q<Tag, D>(w.q[1], q_src, p.q.sn, row0 + 32, p.N, lane);
+                flash2::prescale_q<Tag, D>(w.q[0], p.scale_log2e);
+                flash2::prescale_q<Tag, D>(w.q[1], p.scale_log2e);
+                const int lane_o = flash2::opaque_lane(lane);
+                const int half = lane_o >> 5, n = lane_o & 31;
+                Pipe::second_pair(w, sn, s_ka(par), lane, [&](int qb, int kb, int r) {
+                    // i - j <= W  with  i = row0 + qb*32 + n,  j = edge_w + kb*32 + key:  qb*32 + n <= kb*32 + key
+                    return qb * 32 + n <= kb * 32 + flash::key_of_reg(r, half);
+                });
+            }
+        }
+    };
+    auto k_tile_of_wave = [&](int u, int par) { return wave_reads_c(u) ? s_kc(par) : s_ka(par); };
     const typename Pipe::TileRequest no_req{nullptr, 0};
 
-    // first tile: scores, masks, row maxima (nothing to overlap with yet)
-    request_k(0, 0);
+    // first tile: scores, masks, row maxima (nothing to overlap with yet).  Buffer parity follows u - u0.
     flash::wait_tile_loads();
     __syncthreads();
-    if (n_iter > 1) request_k(1, 1);
-    copy_v(s_v(0), 0);
-    Pipe::k_head(kf, k_tile_of_wave(0, 0), lane);
+    Pipe::k_head(kf, k_tile_of_wave(u0, 0), lane);
     Pipe::template score_phase<true, false, false, false>(w, s_even, kf, s_odd, vf, 0u, lane, kd_c, no_req, vd, no_req);
-    mask_tile(s_even, 0);
+    finish_scores(s_even, u0, 0);
     Pipe::template pv_phase<false, true>(w, vf, s_odd, s_even, mx);
 
     // Row addresses of this wave's share of the tiles the main loop requests next: K tile u + 2, V tile u + 1.
     const int64_t kc_step = (int64_t)kBN * p.kc.sn * 2, ka_step = (int64_t)kBN * p.ka.sn * 2, v_step = (int64_t)kBN * p.v.sn * 2;
-    const char* kc_rows = reinterpret_cast<const char*>(kc + (int64_t)(2 * kBN + wave * KDma::kRowsPerWave) * p.kc.sn);
-    const char* ka_rows = reinterpret_cast<const char*>(ka + (int64_t)(2 * kBN + wave * KDma::kRowsPerWave) * p.ka.sn);
-    const char* v_rows = reinterpret_cast<const char*>(v_src + (int64_t)(kBN + wave * VDma::kRowsPerWave) * p.v.sn);
+    const int r2 = (u0 + 2) * kBN + wave * KDma::kRowsPerWave;
+    const char* kc_rows = reinterpret_cast<const char*>(kc + (int64_t)r2 * p.kc.sn);
+    const char* ka_rows = reinterpret_cast<const char*>(ka + (int64_t)r2 * p.ka.sn);
+    const char* v_rows = reinterpret_cast<const char*>(v_src + (int64_t)(r2 - kBN) * p.v.sn);
     // Iteration u finishes tile u (exponentials, P.V) and prepares tile u + 1 (scores, masks, row maxima); K(u+1) and
     // V(u) were requested one iteration earlier and sit in the buffers of parity u + 1 and u.  It requests K(u+2) and
     // V(u+1): whole tiles ride on the score MFMAs (kRide), anything else goes out as a block in front of them.
@@ -188,19 +262,30 @@ __global__ __launch_bounds__(flash2::kThreads, 1) void prefill_pipe_kernel(Param
         Scores& sn = par ? s_even : s_odd;
         flash::wait_tile_loads();
         __syncthreads();  // K(u+1) and V(u) are complete; every wave is done with K(u) and V(u-1)
+        if constexpr (kSlotsC == 1) {
+            // the one second-source slot is free now: the tile about to be scored is brought and waited for (once or
+            // twice per query tile; the other workgroup of the CU computes meanwhile)
+            if (needs_c(u + 1)) {  // (workgroup-uniform)
+                copy_k(s_kc(0), kc, p.kc.sn, (u + 1) * kBN);
+                flash::wait_tile_loads();
+                __syncthreads();
+            }
+        }
         Pipe::k_head(kf, k_tile_of_wave(u + 1, par + 1), lane);
         typename Pipe::TileRequest kr = no_req, vr = no_req;
         KDma kd = kd_c;
         if constexpr (kRide) {
             const int n2 = (u + 2) * kBN;
-            const bool far = needs_far(u + 2);
-            kr.rows = far ? kc_rows : ka_rows;
-            kr.lds = KDma::lds_of_wave(far ? s_kc(par) : s_ka(par), wave);
+            // the source every wave may need rides; where some waves need the other one too, it follows as a block
+            const bool ride_c = KIND == kVq && needs_c(u + 2);
+            kr.rows = ride_c ? kc_rows : ka_rows;
+            kr.lds = KDma::lds_of_wave(ride_c ? s_kc(par) : s_ka(par), wave);
 #pragma unroll
-            for (int i = 0; i < KDma::kInstr; ++i) kd.off[i] = far ? kd_c.off[i] : kd_a.off[i];
+            for (int i = 0; i < KDma::kInstr; ++i) kd.off[i] = ride_c ? kd_c.off[i] : kd_a.off[i];
             vr.rows = v_rows;
             vr.lds = VDma::lds_of_wave(s_v(par + 1), wave);
-            if (far && needs_exact(u + 2)) copy_k(s_ka(par), ka, p.ka.sn, n2);  // boundary tile: both sources
+            if (KIND == kVq && ride_c && needs_a(u + 2)) copy_k(s_ka(par), ka, p.ka.sn, n2);
+            if (KIND == kRerope && kSlotsC == 2 && needs_c(u + 2)) copy_k(s_kc(par), kc, p.kc.sn, n2);
             kc_rows += kc_step, ka_rows += ka_step, v_rows += v_step;
         } else {
             if (u + 2 < n_iter) request_k(u + 2, par);
@@ -208,12 +293,12 @@ __global__ __launch_bounds__(flash2::kThreads, 1) void prefill_pipe_kernel(Param
         }
         Pipe::update_max(w, mx, sc);
         Pipe::template score_phase<true, true, true, kRide>(w, sn, kf, sc, vf, s_v(par), lane, kd, kr, vd, vr);
-        mask_tile(sn, u + 1);
+        finish_scores(sn, u + 1, par + 1);
         mx[0] = mx[1] = -INFINITY;
         Pipe::template pv_phase<true, true>(w, vf, sc, sn, mx);
     };
     // main loop: pairs of iterations whose requests are whole tiles; then the last few, which may run over the end
-    int u = 0;
+    int u = u0;
     for (; u + 3 < n_whole; u += 2) {
         iteration(std::false_type{}, std::true_type{}, u);
         iteration(std::true_type{}, std::true_type{}, u + 1);
@@ -223,35 +308,54 @@ __global__ __launch_bounds__(flash2::kThreads, 1) void prefill_pipe_kernel(Param
         if (u + 1 < n_iter) iteration(std::true_type{}, std::false_type{}, u + 1);
     }
 
+    // the output rows leave through LDS (every wave its own part of the tile buffers) once no wave reads tiles any more
+    __syncthreads();
+    static_assert((size_t)NW * Pipe::kStoreBytes <= lds_bytes<D, KIND>(), "staging area exceeds the tile buffers");
     Pipe::store(w, p.out + b * p.o_sb + h * p.o_sh, p.o_sn, p.lse ? p.lse + (int64_t)bh * p.N : nullptr, row0, p.N,
-                lane);
+                lane, smem + wave * Pipe::kStoreBytes);
     }
 }
 
-template <typename Tag, int D>
+template <typename Tag, int D, int KIND>
 int launch(Params p, int B, hipStream_t stream) {
     // more than the 64 KB of LDS a launch gets by default: raised once per device and instantiation
-    static bool raised[64] = {};
+    static std::mutex mu;
+    static bool raised[kMaxDevices] = {};
     int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return VQA_ERR_LAUNCH_FAILED;
-    if (!raised[dev]) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_pipe_kernel<Tag, D>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes<D>()) != hipSuccess) {
-            (void)hipGetLastError();
-            return VQA_ERR_LAUNCH_FAILED;
+    const int rc = device_of_pointer(p.q.p, &dev);
+    if (rc != VQA_OK) return rc;
+    {
+        std::lock_guard<std::mutex> lock(mu);
+        if (!raised[dev]) {
+            if (hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_pipe_kernel<Tag, D, KIND>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes<D, KIND>()) != hipSuccess) {
+                (void)hipGetLastError();
+                return VQA_ERR_LAUNCH_FAILED;
+            }
+            raised[dev] = true;
         }
-        raised[dev] = true;
     }
+    constexpr int kBM = waves_of<KIND>() * flash2::kWaveRows;
     const int n_tiles = (p.N + kBM - 1) / kBM;
-    p.pair_tiles = (p.causal && (int64_t)(n_tiles / 2) * B * p.H >= 512) ? 1 : 0;
+    // causal work grows with the query tile: late and early tiles are paired once there are enough workgroups
+    p.pair_tiles = (KIND == kVq && p.causal && (int64_t)(n_tiles / 2) * B * p.H >= 512) ? 1 : 0;
     const dim3 grid(p.pair_tiles ? (n_tiles + 1) / 2 : n_tiles, B * p.H);
-    hipLaunchKernelGGL((prefill_pipe_kernel<Tag, D>), grid, dim3(flash2::kThreads), lds_bytes<D>(), stream, p);
+    constexpr size_t kLds = lds_bytes<D, KIND>();
+    hipLaunchKernelGGL((prefill_pipe_kernel<Tag, D, KIND>), grid, dim3(kBM), kLds, stream, p);
     return launch_status();
+}
+
+template <typename Tag, int KIND>
+int launch_d(const Params& p, int B, int D, hipStream_t stream) {
+    if (D == 64) return launch<Tag, 64, KIND>(p, B, stream);
+    if (D == 128) return launch<Tag, 128, KIND>(p, B, stream);
+    return VQA_ERR_UNSUPPORTED_HEAD_DIM;
 }
 
 }  // namespace pipe
 
-// entry used by vqa_prefill_* (vqa_window.hip) once its arguments are validated and K_hat is written
+// entries used by vqa_prefill_* and vqa_local_attn_* (vqa_window.hip) once their arguments are validated (and K_hat
+// is written)
 namespace flash {
 
 bool prefill_pipe_applies(int window, int boundary_is_block, bool has_exact, bool has_second_pair) {
@@ -260,29 +364,56 @@ bool prefill_pipe_applies(int window, int boundary_is_block, bool has_exact, boo
     return boundary_is_block && window % pipe::kBlock == 0;
 }
 
+// sliding-window kinds: window_rule 0 = strict (j >= i - W), 1 = block rule, 2 = block rule with the ReRoPE pair
+bool window_pipe_applies(int window, int N) { return window > 0 && window % pipe::kBlock == 0 && window < N; }
+
 template <typename Tag>
 int prefill_pipe_run(const View& q, const View& ka, const View& kc, const View& v, uint16_t* out, int64_t o_sb,
                      int64_t o_sh, int64_t o_sn, float* lse, int B, int H, int N, int D, int window, int causal,
                      bool all_far, float scale_log2e, hipStream_t stream) {
     pipe::Params p;
-    p.q = q, p.ka = ka, p.kc = kc, p.v = v;
+    p.q = q, p.q2 = q, p.ka = ka, p.kc = kc, p.v = v;
     p.out = out;
     p.o_sb = o_sb, p.o_sh = o_sh, p.o_sn = o_sn;
     p.lse = lse;
     p.H = H, p.N = N, p.window = window;
     p.causal = causal;
     p.all_far = all_far ? 1 : 0;
+    p.strict = 0;
     p.pair_tiles = 0;
     p.scale_log2e = scale_log2e;
-    if (D == 64) return pipe::launch<Tag, 64>(p, B, stream);
-    if (D == 128) return pipe::launch<Tag, 128>(p, B, stream);
-    return VQA_ERR_UNSUPPORTED_HEAD_DIM;
+    return pipe::launch_d<Tag, pipe::kVq>(p, B, D, stream);
+}
+
+template <typename Tag>
+int window_pipe_run(const View& q1, const View& q2, const View& k1, const View& k2, const View& v, uint16_t* out,
+                    int64_t o_sb, int64_t o_sh, int64_t o_sn, float* lse, int B, int H, int N, int D, int window,
+                    int window_rule, float scale_log2e, hipStream_t stream) {
+    pipe::Params p;
+    p.q = q1, p.q2 = q2, p.ka = k1, p.kc = k2, p.v = v;
+    p.out = out;
+    p.o_sb = o_sb, p.o_sh = o_sh, p.o_sn = o_sn;
+    p.lse = lse;
+    p.H = H, p.N = N, p.window = window;
+    p.causal = 1;
+    p.all_far = 0;
+    p.strict = window_rule == 0 ? 1 : 0;
+    p.pair_tiles = 0;
+    p.scale_log2e = scale_log2e;
+    if (window_rule == 2) return pipe::launch_d<Tag, pipe::kRerope>(p, B, D, stream);
+    return pipe::launch_d<Tag, pipe::kWindow>(p, B, D, stream);
 }
 
 template int prefill_pipe_run<bf16_tag>(const View&, const View&, const View&, const View&, uint16_t*, int64_t, int64_t,
                                         int64_t, float*, int, int, int, int, int, int, bool, float, hipStream_t);
 template int prefill_pipe_run<f16_tag>(const View&, const View&, const View&, const View&, uint16_t*, int64_t, int64_t,
                                        int64_t, float*, int, int, int, int, int, int, bool, float, hipStream_t);
+template int window_pipe_run<bf16_tag>(const View&, const View&, const View&, const View&, const View&, uint16_t*,
+                                       int64_t, int64_t, int64_t, float*, int, int, int, int, int, int, float,
+                                       hipStream_t);
+template int window_pipe_run<f16_tag>(const View&, const View&, const View&, const View&, const View&, uint16_t*,
+                                      int64_t, int64_t, int64_t, float*, int, int, int, int, int, int, float,
+                                      hipStream_t);
 
 }  // namespace flash
 }  // namespace vqa

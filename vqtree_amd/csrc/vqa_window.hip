@@ -493,6 +493,12 @@ template <typename Tag>
 int prefill_pipe_run(const View& q, const View& ka, const View& kc, const View& v, uint16_t* out, int64_t o_sb,
                      int64_t o_sh, int64_t o_sn, float* lse, int B, int H, int N, int D, int window, int causal,
                      bool all_far, float scale_log2e, hipStream_t stream);
+// the same core for the sliding-window modes (window_rule = Mode 0 / 1 / 2) with a window that is a multiple of 128
+bool window_pipe_applies(int window, int N);
+template <typename Tag>
+int window_pipe_run(const View& q1, const View& q2, const View& k1, const View& k2, const View& v, uint16_t* out,
+                    int64_t o_sb, int64_t o_sh, int64_t o_sn, float* lse, int B, int H, int N, int D, int window,
+                    int window_rule, float scale_log2e, hipStream_t stream);
 
 template <typename Tag>
 int local_attn(const void* q1, const void* q2, const void* k1, const void* k2, const void* v, void* out, float* lse,
@@ -525,6 +531,18 @@ int local_attn(const void* q1, const void* q2, const void* k1, const void* k2, c
         const int cover = (N + kTile - 1) / kTile * kTile;  // a multiple of 128 that is >= N
         return prefill_pipe_run<Tag>(p.qa, p.ka, p.ka, p.v, p.out, p.o_sb, p.o_sh, p.o_sn, p.lse, B, H, N, D, cover, 1,
                                      false, p.scale_log2e, stream);
+    }
+    // Sliding windows: the pipelined core (128-row query tiles, two workgroups per CU) where it is the faster one.  A
+    // query tile meets (W + 128) / 64 key tiles, and a workgroup's start and end (cold first tiles and queries, output
+    // rows) are not overlapped with anything on its SIMDs, so it needs long windows: measured over batch x heads
+    // 8 - 128, 2k - 32k tokens, windows 128 - 2048 it takes 0.77 - 0.99 of the tiled kernel's time from W = 1024 on
+    // with at least 2048 workgroups, 1.03 - 1.47 below.
+    if (mode <= kLocalRerope && window_pipe_applies(window, N) && (D == 64 || D == 128) && window >= 1024 &&
+        (int64_t)((N + 127) / 128) * B * H >= 2048) {
+        const int rc = validate(p, B, D);
+        if (rc != VQA_OK) return rc;
+        return window_pipe_run<Tag>(p.qa, p.qb, p.ka, p.kb, p.v, p.out, p.o_sb, p.o_sh, p.o_sn, p.lse, B, H, N, D,
+                                    window, mode, p.scale_log2e, stream);
     }
     return run<Tag>(p, B, D, mode, stream);
 }
