@@ -74,6 +74,33 @@ def test_window_modes(mode, B, H, N, D, W):
         assert_close_lse(lse, want_lse)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("mode", ["strict", "loose", "rerope"])
+@pytest.mark.parametrize("N,D,W", [(4096, 128, 1024), (4000, 128, 1152), (4096, 64, 2048)])
+def test_window_modes_on_the_pipelined_core(mode, N, D, W, dtype):
+    """64 (batch, head) units x >= 4000 tokens with a window of >= 1024 keys that is a multiple of 128: here
+    vqa_local_attn_* runs the sliding-window kinds of the pipelined core (128-row workgroups; for ReRoPE the second
+    pair through a change of the query operand at each wave's window-edge tile).  Three units against the oracle."""
+    _say(f"window on the pipelined core {mode} N{N} D{D} W{W} {dtype}")
+    B, H = 2, 32
+    g = torch.Generator(device="cuda").manual_seed(53)
+    q, k, v, q2, k2 = (torch.randn(B, N, H, D, generator=g, device="cuda").to(dtype) for _ in range(5))
+    if mode == "strict":
+        out, lse = triton_fused_local_attn.flash_attn_func(q, k, v, W), None
+    elif mode == "loose":
+        out, lse = triton_fused_local_attn2.flash_attn_func(q, k, v, W, return_lse=True)
+    else:
+        out, lse = triton_fused_local_attn_rerope.flash_attn_func(q, q2, k, k2, v, W, return_lse=True)
+    torch.cuda.synchronize()
+    for b, h in ((0, 0), (1, 17), (1, 31)):
+        one = lambda x: x[b:b + 1, :, h:h + 1].transpose(1, 2).cpu()
+        want, want_lse = oracle.local_attn(one(q), one(k), one(v), W, mode, None, q2=one(q2), k2=one(k2))
+        assert_close_16(one(out), want, f"{mode} unit ({b},{h})")
+        if lse is not None:
+            # the query operand is scaled by softmax_scale * log2(e) before the products: one more 16-bit rounding
+            assert_close_lse(lse[b:b + 1, h:h + 1], want_lse, atol=1e-2 if dtype == torch.bfloat16 else 2e-3)
+
+
 def test_full_window_causal_attention_at_a_large_shape():
     """A window that covers the sequence is plain causal attention; at 64 heads x 4096 tokens the library runs it on
     the pipelined schedule.  Strict and loose windows are then the same function: checked against each other, against
