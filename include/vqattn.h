@@ -282,6 +282,23 @@ int vqa_decode_devlen_f16(const void* q, const uint8_t* codes, const void* codeb
                           int K, const int64_t* strides, float sm_scale, int num_splits, const int32_t* n_keys_dev,
                           vqa_stream_t stream);
 
+/* vqa_decode for a query that has not been rotated yet: rope_cos / rope_sin are ONE row [D] each of the rotary tables
+ * (the row of the position every coded key sees the query at: the clamped ReRoPE position window + 1), 16-byte
+ * aligned, and the lookup-table kernel rotates the query as it reads it,
+ *     q' = q * cos + rotate_half(q) * sin,  every product and the sum rounded to the element type,
+ * bit for bit what vqa_rope_* writes, so a generation step needs no rotary launch for its query.  n_keys_dev as in
+ * vqa_decode_devlen_* or NULL (then N_max keys are attended).  Counterpart in the reference: the rotation of the
+ * query to `window_length + 1` in front of its (non-functional) seqlen_q == 1 branch, ops/attn_vq.py:445-479. */
+int vqa_decode_roped_bf16(const void* q, const void* rope_cos, const void* rope_sin, const uint8_t* codes,
+                          const void* codebooks, const void* v, void* out, float* lse, void* workspace,
+                          size_t workspace_bytes, int B, int H, int N_max, int D, int M, int K, const int64_t* strides,
+                          float sm_scale, int num_splits, const int32_t* n_keys_dev, vqa_stream_t stream);
+
+int vqa_decode_roped_f16(const void* q, const void* rope_cos, const void* rope_sin, const uint8_t* codes,
+                         const void* codebooks, const void* v, void* out, float* lse, void* workspace,
+                         size_t workspace_bytes, int B, int H, int N_max, int D, int M, int K, const int64_t* strides,
+                         float sm_scale, int num_splits, const int32_t* n_keys_dev, vqa_stream_t stream);
+
 /* vqa_decode_bf16 for callers that cannot allocate or hand over device memory (code under HIP graph capture, tight
  * serving loops, harnesses that forbid hipMalloc): no workspace argument, the lookup table and the split states live
  * in a fixed VQA_DECODE_STATIC_SCRATCH_BYTES array inside the library, one copy per GPU, held until the process ends.

@@ -106,6 +106,61 @@ def test_full_size_sampled_units():
         assert_close_lse(lse[b:b + 1, h:h + 1], want_lse)
 
 
+def test_harness_layer_shape_with_default_splits():
+    """The per-layer shape of the 32-layer decode harness (B4 H32 N65536 D128 M4: 128 units, so the default split
+    count is above one and the merge kernel runs): sampled (b, h) units against the oracle, and a call with one split
+    per unit (direct store, no merge) agrees beyond rounding."""
+    from vqtree_amd import _lib
+
+    B, H, N, D, M = 4, 32, 65536, 128, 4
+    print(f"decode at the harness layer shape B{B} H{H} N{N}", flush=True)
+    assert _lib.load().vqa_decode_default_splits(B, H, N) > 1
+    case = decode_case(B, H, N, D, M, device="cuda", seed=31, on_device=True)
+    out, lse = attn_vq_decode(case.q, case.codes, case.codebooks, case.v, return_lse=True)
+    one = attn_vq_decode(case.q, case.codes, case.codebooks, case.v, num_splits=1)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out.float()).all() and torch.isfinite(lse).all()
+    assert (out.float() - one.float()).abs().max() <= 2e-3
+    for b, h in [(0, 0), (1, 9), (3, 31), (2, 20)]:
+        cpu = lambda t: t.cpu()
+        want, want_lse = oracle.attn_vq_decode(cpu(case.q[b:b + 1, h:h + 1]), cpu(case.codes[b:b + 1, h:h + 1]),
+                                               cpu(case.codebooks[h:h + 1]), cpu(case.v[b:b + 1, h:h + 1]),
+                                               case.softmax_scale)
+        assert_close_16(out[b:b + 1, h:h + 1], want, f"unit {b},{h}")
+        assert_close_lse(lse[b:b + 1, h:h + 1], want_lse)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,H,N,D,M", [(3, 4, 700, 128, 4), (17, 2, 300, 64, 2), (1, 1, 64, 128, 1)])
+def test_query_rotated_inside_the_table_kernel(dtype, B, H, N, D, M):
+    """rope=(cos_row, sin_row): the lookup-table kernel rotates the raw query itself.  The table it builds must be the
+    one built from a query rotated by the rotary kernel beforehand, so the two calls agree bit for bit; the rotated
+    query is also pinned against the oracle's operator-by-operator expression, and the result against the oracle."""
+    from vqtree_amd.ops.attn_vq import apply_rope, rope_tables
+
+    print(f"decode with the rotary folded in: {dtype} B{B} H{H} N{N} D{D} M{M}", flush=True)
+    case = decode_case(B, H, N, D, M, device="cuda", seed=33, dtype=dtype)
+    pos = 257
+    cos, sin = rope_tables(D, 400, dtype=dtype, device="cuda")
+    q_rot = apply_rope(case.q, cos, sin, pos)
+    want_rot = oracle.apply_rope(case.q.cpu(), cos.cpu(), sin.cpu(), pos)
+    assert torch.equal(q_rot.cpu(), want_rot)
+    ref, ref_lse = attn_vq_decode(q_rot, case.codes, case.codebooks, case.v, return_lse=True)
+    got, got_lse = attn_vq_decode(case.q, case.codes, case.codebooks, case.v, return_lse=True, rope=(cos[pos], sin[pos]))
+    torch.cuda.synchronize()
+    assert torch.equal(got, ref) and torch.equal(got_lse, ref_lse)
+    want, want_lse = oracle.attn_vq_decode(want_rot, case.codes.cpu(), case.codebooks.cpu(), case.v.cpu(),
+                                           case.softmax_scale)
+    assert_close_16(got, want, "decode with the rotary folded in")
+    assert_close_lse(got_lse, want_lse)
+    # with the key count in device memory (the recorded-step form)
+    n_sub = N - N // 3
+    n_dev = torch.tensor([n_sub], dtype=torch.int32, device="cuda")
+    got2 = attn_vq_decode(case.q, case.codes, case.codebooks, case.v, rope=(cos[pos], sin[pos]), n_keys=n_dev)
+    ref2 = attn_vq_decode(q_rot, case.codes[:, :, :n_sub], case.codebooks, case.v[:, :, :n_sub])
+    assert (got2.float() - ref2.float()).abs().max() <= 2e-3
+
+
 # ------------------------------------------------------------------ exact-key decode
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("B,H,N,D", [(2, 3, 1000, 128), (1, 2, 1, 128), (1, 1, 63, 64), (2, 2, 64, 128), (1, 2, 65, 64),

@@ -23,6 +23,8 @@ SIGNATURES = {
     "vqa_decode_static_bf16": (c_int, [_P] * 6 + [c_int] * 6 + [_STRIDES, c_float, c_int, _P]),
     "vqa_decode_devlen_bf16": (c_int, [_P] * 7 + [c_size_t] + [c_int] * 6 + [_STRIDES, c_float, c_int, _P, _P]),
     "vqa_decode_devlen_f16": (c_int, [_P] * 7 + [c_size_t] + [c_int] * 6 + [_STRIDES, c_float, c_int, _P, _P]),
+    "vqa_decode_roped_bf16": (c_int, [_P] * 9 + [c_size_t] + [c_int] * 6 + [_STRIDES, c_float, c_int, _P, _P]),
+    "vqa_decode_roped_f16": (c_int, [_P] * 9 + [c_size_t] + [c_int] * 6 + [_STRIDES, c_float, c_int, _P, _P]),
     "vqa_decode_windowed_workspace_bytes": (c_size_t, [c_int] * 6),
     "vqa_decode_windowed_bf16": (c_int, [_P] * 9 + [c_size_t] + [c_int] * 7 + [_STRIDES, c_float, _P]),
     "vqa_decode_windowed_f16": (c_int, [_P] * 9 + [c_size_t] + [c_int] * 7 + [_STRIDES, c_float, _P]),

@@ -32,10 +32,51 @@ struct Strides {
 //    C[code, b] = sum_d cb[code, d] * q[b, d] as D/32 MFMA 16x16x32 steps; A and B fragments come straight from
 //    global memory (each lane: 8 contiguous elements of its row).
 // ---------------------------------------------------------------------------------------------------------------
+//    With rope_cos / rope_sin (one [D] row each: the tables at the query's position) the query is rotated on the way in,
+//    q' = q * cos + rotate_half(q) * sin with every product and the sum rounded to the element type -- bit for bit what
+//    the rotary kernel (vqa_rope.hip) writes -- so a caller with an unrotated query needs no launch for it.
+template <typename Tag>
+__device__ __forceinline__ float rnd16(float x) { return Elem<Tag>::round_keep_f32(x); }
+
+// one 8-element slice of the rotated query: x = the slice itself, xp = its rotate_half partner (D/2 elements away),
+// c / s = the cos / sin slices at x's place; upper = x lies in the upper half of the row
+template <typename Tag>
+__device__ __forceinline__ typename Elem<Tag>::vec8 rotate_slice(typename Elem<Tag>::vec8 x, typename Elem<Tag>::vec8 xp,
+                                                                 typename Elem<Tag>::vec8 c, typename Elem<Tag>::vec8 s,
+                                                                 bool upper) {
+// every product and the sum round on their own: no fused multiply-add (for f16 the compiler turns the conversions below
+// into 16-bit arithmetic, which it would then contract)
+#pragma clang fp contract(off)
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    const u32x4 xw = __builtin_bit_cast(u32x4, x), pw = __builtin_bit_cast(u32x4, xp);
+    const u32x4 cw = __builtin_bit_cast(u32x4, c), sw = __builtin_bit_cast(u32x4, s);
+    u32x4 o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        uint32_t pair = 0;
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const int sh = 16 * t;
+            const float xv = Elem<Tag>::from_bits((uint16_t)(xw[e] >> sh)), pv = Elem<Tag>::from_bits((uint16_t)(pw[e] >> sh));
+            const float cv = Elem<Tag>::from_bits((uint16_t)(cw[e] >> sh)), sv = Elem<Tag>::from_bits((uint16_t)(sw[e] >> sh));
+            // lower half: x*cos + (-partner)*sin; upper half: x*cos + partner*sin (products of two 16-bit values are
+            // exact in fp32, so each rounding below is the only one of its operator)
+            // (rounding is symmetric: subtracting the rounded product is adding the rounded negated one)
+            const float t0 = rnd16<Tag>(xv * cv), t1 = rnd16<Tag>(pv * sv);
+            const float r = rnd16<Tag>(upper ? t0 + t1 : t0 - t1);
+            pair |= (uint32_t)Elem<Tag>::to_bits(r) << sh;
+        }
+        o[e] = pair;
+    }
+    return __builtin_bit_cast(typename Elem<Tag>::vec8, o);
+}
+
 template <typename Tag, int D>
 __global__ __launch_bounds__(kThreads) void lut_kernel(const uint16_t* __restrict__ q,
                                                        const uint16_t* __restrict__ cb, float* __restrict__ lut,
-                                                       int B, int H, int M, int K, Strides st, float scale_log2e) {
+                                                       int B, int H, int M, int K, Strides st, float scale_log2e,
+                                                       const uint16_t* __restrict__ rope_cos,
+                                                       const uint16_t* __restrict__ rope_sin) {
     typedef typename Elem<Tag>::vec8 vec8;
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -57,11 +98,23 @@ __global__ __launch_bounds__(kThreads) void lut_kernel(const uint16_t* __restric
         const int bb = b0 + r;
         f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
         const uint16_t* b_row = q + (int64_t)min(bb, B - 1) * st.q_b + h * st.q_h + kq * 8;
+        vec8 bv[D / 32];
 #pragma unroll
-        for (int kk = 0; kk < D / 32; ++kk) {
-            vec8 bv = *reinterpret_cast<const vec8*>(b_row + kk * 32);
-            acc = Elem<Tag>::mfma16(a[kk], bv, acc);
+        for (int kk = 0; kk < D / 32; ++kk) bv[kk] = *reinterpret_cast<const vec8*>(b_row + kk * 32);
+        if (rope_cos != nullptr) {  // (uniform)
+            vec8 rv[D / 32];
+#pragma unroll
+            for (int kk = 0; kk < D / 32; ++kk) {
+                constexpr int kHalf = D / 64;  // slices per half row: the partner of slice kk is kk ^ kHalf
+                const vec8 c = *reinterpret_cast<const vec8*>(rope_cos + kk * 32 + kq * 8);
+                const vec8 sn = *reinterpret_cast<const vec8*>(rope_sin + kk * 32 + kq * 8);
+                rv[kk] = rotate_slice<Tag>(bv[kk], bv[kk ^ kHalf], c, sn, kk >= kHalf);
+            }
+#pragma unroll
+            for (int kk = 0; kk < D / 32; ++kk) bv[kk] = rv[kk];
         }
+#pragma unroll
+        for (int kk = 0; kk < D / 32; ++kk) acc = Elem<Tag>::mfma16(a[kk], bv[kk], acc);
         // acc[i]: codeword row 4*kq + i, batch column r
         if (bb < B) {
             float* dst = lut + ((int64_t)(bb * H + h) * M + m) * kLutStride + tile * 16 + kq * 4;
@@ -544,7 +597,8 @@ int launch_main(const uint8_t* codes, const uint16_t* v, const float* lut, float
 template <typename Tag, int D>
 int run_d(const void* q, const uint8_t* codes, const void* codebooks, const void* v, void* out, float* lse,
           void* workspace, int B, int H, int N, int M, int K, const Strides& st, float sm_scale, int S,
-          const int* n_keys_dev, hipStream_t stream) {
+          const int* n_keys_dev, hipStream_t stream, const uint16_t* rope_cos = nullptr,
+          const uint16_t* rope_sin = nullptr) {
     const Workspace ws = plan(B, H, D, M, S);
     char* base = static_cast<char*>(workspace);
     float* lut = reinterpret_cast<float*>(base + ws.lut_off);
@@ -556,7 +610,7 @@ int run_d(const void* q, const uint8_t* codes, const void* codebooks, const void
 
     const int tiles = kLutStride / 16;
     hipLaunchKernelGGL((lut_kernel<Tag, D>), dim3((tiles + kWaves - 1) / kWaves, H * M), dim3(kThreads), 0, stream,
-                       q16, cb16, lut, B, H, M, K, st, sm_scale * kLog2e);
+                       q16, cb16, lut, B, H, M, K, st, sm_scale * kLog2e, rope_cos, rope_sin);
     int rc = launch_status();
     if (rc != VQA_OK) return rc;
 
@@ -612,8 +666,11 @@ inline int static_scratch(void** out) {
 template <typename Tag>
 int run(const void* q, const uint8_t* codes, const void* codebooks, const void* v, void* out, float* lse,
         void* workspace, size_t workspace_bytes, int B, int H, int N, int D, int M, int K, const int64_t* strides,
-        float sm_scale, int num_splits, const int* n_keys_dev, hipStream_t stream) {
+        float sm_scale, int num_splits, const int* n_keys_dev, hipStream_t stream, const void* rope_cos = nullptr,
+        const void* rope_sin = nullptr) {
     if (!q || !codes || !codebooks || !v || !out || !workspace || !strides) return VQA_ERR_NULL_POINTER;
+    if ((rope_cos == nullptr) != (rope_sin == nullptr)) return VQA_ERR_NULL_POINTER;
+    if (!aligned16(rope_cos) || !aligned16(rope_sin)) return VQA_ERR_MISALIGNED;
     if (B <= 0 || H <= 0 || N <= 0) return VQA_ERR_BAD_SHAPE;
     if (D != 64 && D != 128) return VQA_ERR_UNSUPPORTED_HEAD_DIM;
     if ((M != 1 && M != 2 && M != 4 && M != 8) || K < 1 || K > 256) return VQA_ERR_UNSUPPORTED_CODEBOOK;
@@ -632,11 +689,13 @@ int run(const void* q, const uint8_t* codes, const void* codebooks, const void* 
     int S = num_splits > 0 ? num_splits : default_splits(B, H, N);
     if (S > 65535 || (int64_t)B * H > 65535) return VQA_ERR_BAD_ARGUMENT;
     if (workspace_bytes < plan(B, H, D, M, S).total) return VQA_ERR_WORKSPACE_TOO_SMALL;
+    const uint16_t* rc16 = static_cast<const uint16_t*>(rope_cos);
+    const uint16_t* rs16 = static_cast<const uint16_t*>(rope_sin);
     if (D == 64)
         return run_d<Tag, 64>(q, codes, codebooks, v, out, lse, workspace, B, H, N, M, K, st, sm_scale, S, n_keys_dev,
-                              stream);
+                              stream, rc16, rs16);
     return run_d<Tag, 128>(q, codes, codebooks, v, out, lse, workspace, B, H, N, M, K, st, sm_scale, S, n_keys_dev,
-                           stream);
+                           stream, rc16, rs16);
 }
 
 // strides: q(b,h) k(b,h,n) v(b,h,n) out(b,h)
@@ -716,7 +775,7 @@ int run_windowed_d(const uint16_t* q_far, const uint16_t* q_win, const uint8_t* 
     if (far > 0) {
         const int tiles = kLutStride / 16;
         hipLaunchKernelGGL((lut_kernel<Tag, D>), dim3((tiles + kWaves - 1) / kWaves, H * M), dim3(kThreads), 0, stream,
-                           q_far, cb, lut, B, H, M, K, st, sm_scale * kLog2e);
+                           q_far, cb, lut, B, H, M, K, st, sm_scale * kLog2e, nullptr, nullptr);
         if ((rc = launch_status()) != VQA_OK) return rc;
         int kps = ((far + s_far - 1) / s_far + kThreads - 1) / kThreads * kThreads;
         switch (M) {
@@ -882,6 +941,24 @@ int vqa_decode_devlen_f16(const void* q, const uint8_t* codes, const void* codeb
     if (!n_keys_dev) return VQA_ERR_NULL_POINTER;
     return vqa::decode::run<vqa::f16_tag>(q, codes, codebooks, v, out, lse, workspace, workspace_bytes, B, H, N_max, D,
                                           M, K, strides, sm_scale, num_splits, n_keys_dev, stream);
+}
+
+int vqa_decode_roped_bf16(const void* q, const void* rope_cos, const void* rope_sin, const uint8_t* codes,
+                          const void* codebooks, const void* v, void* out, float* lse, void* workspace,
+                          size_t workspace_bytes, int B, int H, int N_max, int D, int M, int K, const int64_t* strides,
+                          float sm_scale, int num_splits, const int32_t* n_keys_dev, vqa_stream_t stream) {
+    if (!rope_cos || !rope_sin) return VQA_ERR_NULL_POINTER;
+    return vqa::decode::run<vqa::bf16_tag>(q, codes, codebooks, v, out, lse, workspace, workspace_bytes, B, H, N_max, D,
+                                           M, K, strides, sm_scale, num_splits, n_keys_dev, stream, rope_cos, rope_sin);
+}
+
+int vqa_decode_roped_f16(const void* q, const void* rope_cos, const void* rope_sin, const uint8_t* codes,
+                         const void* codebooks, const void* v, void* out, float* lse, void* workspace,
+                         size_t workspace_bytes, int B, int H, int N_max, int D, int M, int K, const int64_t* strides,
+                         float sm_scale, int num_splits, const int32_t* n_keys_dev, vqa_stream_t stream) {
+    if (!rope_cos || !rope_sin) return VQA_ERR_NULL_POINTER;
+    return vqa::decode::run<vqa::f16_tag>(q, codes, codebooks, v, out, lse, workspace, workspace_bytes, B, H, N_max, D,
+                                          M, K, strides, sm_scale, num_splits, n_keys_dev, stream, rope_cos, rope_sin);
 }
 
 }  // extern "C"

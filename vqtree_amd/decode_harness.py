@@ -59,7 +59,7 @@ class VQDecodeModel:
         self.kwin_len = 0
         self.cos, self.sin = rope_tables(head_dim, max(capacity, window + 2), dtype=dtype, device=device)
         # every far key is seen at the clamped position
-        self.cos_w, self.sin_w = self.cos[window + 1], self.sin[window + 1]
+        self.cos_w, self.sin_w = self.cos[window + 1].contiguous(), self.sin[window + 1].contiguous()
 
     def fill_random_context(self, n_tokens, seed=6):
         """Synthetic cache contents standing in for a prefill of n_tokens (random codes, V ~ N(0,1))."""
@@ -85,10 +85,14 @@ class VQDecodeModel:
         """Attention of the new token (cache rows [0, n] are filled).  Coded keys are scored with the query at the
         clamped position window + 1, exact window keys with the query at its true position n."""
         scale = 1.0 / math.sqrt(self.D)
-        q_far = apply_rope(q_raw.unsqueeze(2), self.cos, self.sin, self.window + 1)  # [B,H,1,D], one launch
         codes, values = layer["codes"][:, :, : n + 1], layer["values"][:, :, : n + 1]
+        if not self.exact_window and attention is None:
+            # the clamped rotation of the query happens inside the lookup-table kernel
+            return attn_vq_decode(q_raw.unsqueeze(2), codes, layer["codebooks"], values, softmax_scale=scale,
+                                  rope=(self.cos_w, self.sin_w))
+        q_far = apply_rope(q_raw.unsqueeze(2), self.cos, self.sin, self.window + 1)  # [B,H,1,D], one launch
         if not self.exact_window:
-            return (attention or attn_vq_decode)(q_far, codes, layer["codebooks"], values, softmax_scale=scale)
+            return attention(q_far, codes, layer["codebooks"], values, softmax_scale=scale)
         w = min(self.exact_window, n + 1)
         k_win = layer["kwin"][:, :, win_end - w: win_end]
         q_win = (q_raw * self.cos[n] + rotate_half(q_raw) * self.sin[n]).unsqueeze(2)
@@ -158,11 +162,11 @@ class VQDecodeModel:
             h = self._rms(x)
             qkv = (h @ layer["wqkv"]).view(B, 3, H, D)
             q, k, v = qkv[:, 0], qkv[:, 1], qkv[:, 2]
-            q2 = apply_rope(q.unsqueeze(2), self.cos, self.sin, self.window + 1)
             layer["codes"].index_copy_(2, self.pos_dev, encode_residual(k.unsqueeze(2), layer["codebooks"]))
             layer["values"].index_copy_(2, self.pos_dev, v.unsqueeze(2))
-            attn_vq_decode(q2, layer["codes"], layer["codebooks"], layer["values"], softmax_scale=1.0 / math.sqrt(D),
-                           num_splits=self.splits, n_keys=self.n_dev, out=self.attn_out, workspace=self.ws)
+            attn_vq_decode(q.unsqueeze(2), layer["codes"], layer["codebooks"], layer["values"],
+                           softmax_scale=1.0 / math.sqrt(D), num_splits=self.splits, n_keys=self.n_dev,
+                           out=self.attn_out, workspace=self.ws, rope=(self.cos_w, self.sin_w))
             x = x + self.attn_out.reshape(B, H * D) @ layer["wo"]
             h = self._rms(x)
             gate, up = (h @ layer["w_gate_up"]).chunk(2, dim=-1)

@@ -22,7 +22,7 @@ def _last_dim_contiguous(x):
 
 
 def attn_vq_decode(q, k_codes, codebooks, v, *, softmax_scale=None, return_lse=False, num_splits=0, n_keys=None,
-                   out=None, workspace=None):
+                   out=None, workspace=None, rope=None):
     """out[b,h] = softmax_j(scale * sum_m <q[b,h], codebooks[h,m,k_codes[b,h,j,m]]>) @ v[b,h]   (no mask).
 
     q [B,H,1,D] bf16/f16, k_codes [B,H,N,M] uint8, codebooks [H,M,K,D], v [B,H,N,D]  ->  out [B,H,1,D] (q's dtype)
@@ -31,6 +31,10 @@ def attn_vq_decode(q, k_codes, codebooks, v, *, softmax_scale=None, return_lse=F
     `n_keys` (int32 tensor with one element, on the device): the number of keys to attend is read from it when the
     kernels run, N being only the capacity of the buffers -- for launch sequences recorded once (a HIP graph of a decode
     step) and replayed as the cache grows.  `out` / `workspace` let such a caller provide the buffers.
+
+    `rope = (cos_row, sin_row)` (two [D] rows of the rotary tables, q's dtype): q is the UNROTATED query and is rotated
+    to that position inside the lookup-table kernel, with the rounding of `apply_rope` -- the clamped ReRoPE query of a
+    generation step without a launch of its own.
     """
     lib = _lib.load()
     _lib.require_gpu(q, k_codes, codebooks, v)
@@ -64,16 +68,24 @@ def attn_vq_decode(q, k_codes, codebooks, v, *, softmax_scale=None, return_lse=F
         v.stride(0), v.stride(1), v.stride(2),
         out.stride(0), out.stride(1),
     )  # fmt: skip
+    if n_keys is not None:
+        assert n_keys.dtype == torch.int32 and n_keys.numel() == 1 and n_keys.is_cuda
     with torch.cuda.device(q.device):
-        args = (q.data_ptr(), k_codes.data_ptr(), codebooks.data_ptr(), v.data_ptr(), out.data_ptr(),
+        tail = (k_codes.data_ptr(), codebooks.data_ptr(), v.data_ptr(), out.data_ptr(),
                 lse.data_ptr() if return_lse else None,
                 workspace.data_ptr(), ws_bytes, B, H, N, D, M, K, strides, softmax_scale, splits)  # fmt: skip
-        if n_keys is None:
-            rc = getattr(lib, "vqa_decode_" + _SUFFIX[q.dtype])(*args, _lib.current_stream(q.device))
+        stream = _lib.current_stream(q.device)
+        if rope is not None:
+            cos_row, sin_row = (t if t.is_contiguous() else t.contiguous() for t in rope)
+            assert cos_row.shape == sin_row.shape == (D,) and cos_row.dtype == sin_row.dtype == q.dtype
+            _lib.require_gpu(cos_row, sin_row)
+            rc = getattr(lib, "vqa_decode_roped_" + _SUFFIX[q.dtype])(
+                q.data_ptr(), cos_row.data_ptr(), sin_row.data_ptr(), *tail,
+                None if n_keys is None else n_keys.data_ptr(), stream)
+        elif n_keys is None:
+            rc = getattr(lib, "vqa_decode_" + _SUFFIX[q.dtype])(q.data_ptr(), *tail, stream)
         else:
-            assert n_keys.dtype == torch.int32 and n_keys.numel() == 1 and n_keys.is_cuda
-            rc = getattr(lib, "vqa_decode_devlen_" + _SUFFIX[q.dtype])(*args, n_keys.data_ptr(),
-                                                                       _lib.current_stream(q.device))
+            rc = getattr(lib, "vqa_decode_devlen_" + _SUFFIX[q.dtype])(q.data_ptr(), *tail, n_keys.data_ptr(), stream)
         _lib.check(rc)
     return (out, lse) if return_lse else out
 
