@@ -4,16 +4,19 @@
  * This is the boundary a host binds instead of the reference's Triton launches.  Every entry point
  *   - takes plain device pointers, sizes and element strides (no torch types),
  *   - enqueues its kernels on the given HIP stream and returns without synchronising,
- *   - allocates nothing and keeps no mutable global state (scratch comes in through `workspace`; the one exception,
- *     vqa_decode_static_bf16, works in a fixed device array of the library and says so below),
+ *   - allocates nothing and keeps no state between calls (scratch comes in through `workspace`; the one exception,
+ *     vqa_decode_static_bf16, works in a fixed device array of the library and says so below).  What the library does
+ *     remember, behind a mutex, is per-device set-up done on first use: the raised dynamic-LDS limit of the kernels
+ *     that need more than 64 KB (the count kernel at head dim 128, the pipelined prefill / window kernels) and the
+ *     device address of that array.  Both belong to the device that owns the call's operands, which must be the
+ *     calling thread's current device (VQA_ERR_BAD_ARGUMENT otherwise: the kernels would be launched elsewhere),
  *   - returns VQA_OK (0) or a negative vqa_status; it never throws or aborts.
  * Tensors are addressed as base + sum(index_i * stride_i) in ELEMENTS of their own type; the innermost
  * (head_dim / codebook index M) stride must be 1.  Head dims of the attention entry points: 64 and 128; vqa_local_attn_*,
  * vqa_rerope_full_* and vqa_vqcount_* also take 32 (the reference's kernels of these kinds accept 16, 32, 64 and 128,
  * ops/triton_fused_attn_rerope.py:192, ops/triton_fused_vq_attn.py:198-199; a caller with head dim 16 zero-pads its
  * operands to 32, which leaves the scores unchanged, and drops the padded output columns -- the Python layer does).
- * The encoder, preprocessing and rotary entry points state their own limits.  The count kernel needs 64.5 KB of LDS at head dim
- * 128 and raises its dynamic-LDS limit with hipFuncSetAttribute on every call; nothing else touches process state.
+ * The encoder, preprocessing and rotary entry points state their own limits.
  *
  * Log-sum-exp values are base 2 of the scaled scores, lse2 = log2(sum_j exp(s_ij * sm_scale)), the convention of
  * the reference kernels (ops/triton_fused_vq_attn.py:179, ops/triton_fused_local_attn_rerope.py:214-216).
@@ -437,7 +440,7 @@ int vqa_rope_f16(const void* x, const int64_t* position_ids, const void* cos, co
  *
  *   vqa_count_state_add: fold T keys into the state, cnt[b,h,ids[b,h,t]] += 1 and Vsum[b,h,ids[b,h,t],:] += v[b,h,t,:]
  *     (fp32 sums in position order, no atomics: results are reproducible).  ids [B,H,T] int64 (entries outside [0, C)
- *     are skipped), v [B,H,T,D]; cnt [B,H,C] int32 and vsum [B,H,C,D] fp32 contiguous, zeroed by the caller before the
+ *     are clamped into it, as everywhere in this library), v [B,H,T,D]; cnt [B,H,C] int32 and vsum [B,H,C,D] fp32 contiguous, zeroed by the caller before the
  *     first call.  strides[0..5] = ids(b,h,t) v(b,h,t).  D in {64, 128}.
  *   vqa_count_decode: out[b,h,:] = sum_c e_c Vsum[b,h,c,:] / Z with e_c = exp(q[b,h].cb[h,c] * sm_scale) for the
  *     codewords with cnt > 0; lse (nullable, [B,H] fp32) = log2 Z, -inf for an empty state (out = 0) -- the pair is an

@@ -128,9 +128,24 @@ def test_count_state_and_schedule_entry_points_reject_bad_arguments_before_any_l
     assert lib.vqa_vqcount_merge_icnt_bf16(16, 16, 16, 16, 16, 16, None, 1, 1, 512, 128, 128, s17, 128, 1.0, None) == -1
 
 
+def test_roped_decode_rejects_bad_arguments_before_any_launch(lib):
+    strides = _lib.strides_array(*([0] * 12))
+
+    def call(cos=16, sin=16, q=16, D=128):
+        return lib.vqa_decode_roped_bf16(q, cos, sin, 16, 16, 16, 16, None, 256, 1 << 20, 1, 1, 8, D, 4, 256, strides,
+                                         1.0, 1, None, None)
+
+    assert call(cos=None) == -1 and call(sin=None) == -1 and call(q=None) == -1  # VQA_ERR_NULL_POINTER
+    assert call(cos=18) == -5                                                  # VQA_ERR_MISALIGNED
+    assert call(D=96) == -3                                                    # VQA_ERR_UNSUPPORTED_HEAD_DIM
+
+
 def test_static_scratch_decode_refuses_oversized_problem_on_the_host(lib):
     strides = _lib.strides_array(*([0] * 12))
-    rc = lib.vqa_decode_static_bf16(16, 16, 16, 16, 16, None, 16, 32, 1 << 20, 128, 4, 256, strides, 1.0, 64, None)
+    # (NULL tensors: were the size check ever moved behind the others, the call would still stop at the pointer
+    # check and launch nothing)
+    rc = lib.vqa_decode_static_bf16(None, None, None, None, None, None, 16, 32, 1 << 20, 128, 4, 256, strides, 1.0, 64,
+                                    None)
     assert rc == -9 and b"static" in lib.vqa_strerror(rc)
 
 

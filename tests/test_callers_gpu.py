@@ -231,3 +231,74 @@ def test_rerope_caller_routes():
     scores = q1[:, :, :Ns].float().cpu() @ k1[:, :, :Ns].float().cpu().transpose(-1, -2) / math.sqrt(D)
     ref_s, _ = oracle.attend(scores, torch.ones(Ns, Ns, dtype=torch.bool).tril(), v[:, :, :Ns].float().cpu())
     assert_close_16(short.view(B, Ns, H, D).transpose(1, 2).cpu(), ref_s)
+
+
+def _largest_tensor(obj, seen=None):
+    """Largest number of elements of any tensor reachable from obj (attributes, lists, tuples, dicts)."""
+    seen = set() if seen is None else seen
+    if id(obj) in seen:
+        return 0
+    seen.add(id(obj))
+    if torch.is_tensor(obj):
+        return obj.numel()
+    if isinstance(obj, (list, tuple)):
+        return max([_largest_tensor(x, seen) for x in obj] + [0])
+    if isinstance(obj, dict):
+        return max([_largest_tensor(x, seen) for x in obj.values()] + [0])
+    if hasattr(obj, "__dict__"):
+        return _largest_tensor(vars(obj), seen)
+    return 0
+
+
+@pytest.mark.parametrize("exact_window", [False, True])
+def test_cache_keeps_no_tensor_of_the_prefill_size(exact_window):
+    """What the VQ memory is for: after a long prefill (and after a generation step) the cache holds the count state
+    [B,H,C,D], window buffers and one code byte per key -- no [B,H,N,D] tensor, and no closure over one."""
+    import gc
+    import weakref
+
+    B, H, N, D, W, C = 1, 2, 4096, 128, 256, 128
+    q, k, v = _states(B, H, N, D, torch.bfloat16, 41)
+    cb = torch.randn(H, C, D, generator=torch.Generator("cpu").manual_seed(42)).to(torch.bfloat16).cuda()
+    pos = torch.arange(N, device="cuda").unsqueeze(0)
+    cache = A.VectorQuantizedReRoPECache(W, cb, generation_exact_window=exact_window)
+    A.dispatch_attn(q, k, v, pos, cache)
+    limit = B * H * max(C, W + 256) * D  # count-state sums / window buffers; the code bytes are B*H*N
+    assert _largest_tensor(cache) <= max(limit, B * H * N)
+    assert not hasattr(cache, "value_cache")
+    refs = [weakref.ref(t) for t in (k, v)]
+    del q, k, v
+    gc.collect()
+    assert all(r() is None for r in refs), "the cache still references the prefill's keys / values"
+    qs, ks, vs = _states(B, H, 1, D, torch.bfloat16, 43)
+    out = A.dispatch_attn(qs, ks, vs, torch.full((B, 1), N, device="cuda"), cache)
+    torch.cuda.synchronize()
+    assert out.shape == (B, 1, H * D) and torch.isfinite(out.float()).all()
+    assert _largest_tensor(cache) <= max(limit, B * H * (N + 1))
+
+
+def test_long_prefill_route_records_into_a_hip_graph():
+    """The linear-time prefill route makes no device-to-host copy (rotary tables are sized on the host), so it can be
+    recorded once and replayed: every replay must reproduce the eager result bit for bit."""
+    B, H, N, D, W, C = 1, 4, 2048, 128, 512, 256
+    q, k, v = _states(B, H, N, D, torch.bfloat16, 51)
+    cb = torch.randn(H, C, D, generator=torch.Generator("cpu").manual_seed(52)).to(torch.bfloat16).cuda()
+    pos = torch.arange(N, device="cuda").unsqueeze(0)
+    run = lambda: A.dispatch_attn(q, k, v, pos, A.VectorQuantizedReRoPECache(W, cb))
+    eager = run()  # also the warm-up: per-device set-up of the kernels happens outside the capture
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        recorded = run()
+    for i in range(3):
+        recorded.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        _ = (q.float() * 2).sum().item()  # eager work and a synchronisation between the replays
+        torch.cuda.synchronize()
+        assert torch.equal(recorded, eager), f"replay {i}"

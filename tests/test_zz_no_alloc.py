@@ -52,6 +52,9 @@ def test_static_scratch_decode_matches_workspace_decode_twice(lib):
 def test_static_scratch_decode_refuses_oversized_problem(lib):
     # 16 x 32 x 64 splits x (128 + 2) floats of split states alone exceed the 8 MiB array: refused on the host
     strides = _lib.strides_array(*([0] * 12))
-    rc = lib.vqa_decode_static_bf16(16, 16, 16, 16, 16, None, 16, 32, 1 << 20, 128, 4, 256, strides, 1.0, 64, None)
+    # (NULL tensors: were the size check ever moved behind the others, the call would still stop at the pointer
+    # check and launch nothing)
+    rc = lib.vqa_decode_static_bf16(None, None, None, None, None, None, 16, 32, 1 << 20, 128, 4, 256, strides, 1.0, 64,
+                                    None)
     assert rc == -9
     assert b"static" in lib.vqa_strerror(rc)

@@ -3,6 +3,8 @@
 // count kernel: query tile t covers rows [W + T + t*T, W + T + (t+1)*T) and attends over the C codewords of its
 // head: score_c = q2 . codebook[c]; codewords that no key up to block t uses (cnt == 0) are masked; the numerator
 // sums P . v_vq[vi[t, c]] (per-code running sums of V), the denominator weights exp by cnt[t, c].
+#include <mutex>
+
 #include "vqa_flash.h"
 
 namespace vqa {
@@ -170,11 +172,23 @@ __global__ __launch_bounds__(kThreads, 2) void count_kernel(CountParams p) {
 template <typename Tag, int D>
 int launch_count(const CountParams& p, dim3 grid, hipStream_t stream) {
     constexpr size_t kLds = 4 * Geom<D>::kTileBytes + 2 * kBN * sizeof(float);
-    if (kLds > 65536 &&
-        hipFuncSetAttribute(reinterpret_cast<const void*>(&count_kernel<Tag, D>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLds) != hipSuccess) {
-        (void)hipGetLastError();
-        return VQA_ERR_LAUNCH_FAILED;
+    if (kLds > 65536) {
+        // more than the 64 KB of LDS a launch gets by default: raised once per device (the one that owns the
+        // operands, which must be the current one) and instantiation
+        static std::mutex mu;
+        static bool raised[kMaxDevices] = {};
+        int dev = 0;
+        const int rc = device_of_pointer(p.q.p, &dev);
+        if (rc != VQA_OK) return rc;
+        std::lock_guard<std::mutex> lock(mu);
+        if (!raised[dev]) {
+            if (hipFuncSetAttribute(reinterpret_cast<const void*>(&count_kernel<Tag, D>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLds) != hipSuccess) {
+                (void)hipGetLastError();
+                return VQA_ERR_LAUNCH_FAILED;
+            }
+            raised[dev] = true;
+        }
     }
     hipLaunchKernelGGL((count_kernel<Tag, D>), grid, dim3(kThreads), kLds, stream, p);
     return launch_status();

@@ -50,9 +50,12 @@ __global__ __launch_bounds__(D) void add_kernel(const int64_t* __restrict__ ids,
     for (int t0 = 0; t0 < T; t0 += D) {
         // order-preserving compaction of the chunk's keys that belong to this group
         const int t = t0 + tid;
-        const int64_t id = t < T ? my_ids[t * i_st] : -1;
+        // an id outside [0, C) counts as the nearest valid codeword, the rule of every kernel that reads ids or codes
+        // (preprocessing, key reconstruction, lookup table): the state then matches the prefill of the same cache
+        const int64_t raw = t < T ? my_ids[t * i_st] : 0;
+        const int64_t id = raw < 0 ? 0 : (raw >= C ? C - 1 : raw);
         const int64_t rel = id - c0;
-        const bool mine = rel >= 0 && rel < kCodesPerGroup && id < C;
+        const bool mine = t < T && rel >= 0 && rel < kCodesPerGroup;
         const uint64_t mask = __builtin_amdgcn_ballot_w64(mine);
         if (lane == 0) s_wave_n[wave] = __builtin_popcountll(mask);
         __syncthreads();

@@ -640,16 +640,14 @@ int run_d(const void* q, const uint8_t* codes, const void* codebooks, const void
 // ---------------------------------------------------------------------------------------------------------------
 static __device__ __align__(256) unsigned char scratch[VQA_DECODE_STATIC_SCRATCH_BYTES];
 
-constexpr int kMaxDevices = 64;
-
-inline int static_scratch(void** out) {
+// `operand`: a device pointer of the call; the scratch copy used is the one of the device that owns it, which must be
+// the calling thread's current device (the launches that follow run there)
+inline int static_scratch(const void* operand, void** out) {
     static std::mutex mu;
     static void* ptrs[kMaxDevices] = {};
     int dev = -1;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
-        (void)hipGetLastError();
-        return VQA_ERR_LAUNCH_FAILED;
-    }
+    const int rc = device_of_pointer(operand, &dev);
+    if (rc != VQA_OK) return rc;
     std::lock_guard<std::mutex> lock(mu);
     if (ptrs[dev] == nullptr) {
         void* ptr = nullptr;
@@ -919,7 +917,7 @@ int vqa_decode_static_bf16(const void* q, const uint8_t* codes, const void* code
     const int S = num_splits > 0 ? num_splits : vqa::decode::default_splits(B, H, N);
     if (vqa::decode::plan(B, H, D, M, S).total > (size_t)VQA_DECODE_STATIC_SCRATCH_BYTES) return VQA_ERR_SCRATCH_LIMIT;
     void* ws = nullptr;
-    const int rc = vqa::decode::static_scratch(&ws);
+    const int rc = vqa::decode::static_scratch(q, &ws);
     if (rc != VQA_OK) return rc;
     return vqa::decode::run<vqa::bf16_tag>(q, codes, codebooks, v, out, lse, ws, VQA_DECODE_STATIC_SCRATCH_BYTES, B, H,
                                            N, D, M, K, strides, sm_scale, S, nullptr, stream);

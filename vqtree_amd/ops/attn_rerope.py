@@ -94,7 +94,8 @@ def rerope_attn_forward(query_states, key_states, value_states, position_ids, ca
     past = cache.get_seq_length(layer_idx)
     assert past == 0 or q_len == 1, "Only support prefilling or generation"
     scale = 1.0 / math.sqrt(D)
-    n_pos = max(past + q_len, int(position_ids.max()) + 1, W + 1, 2)
+    # sized on the host (no device-to-host copy of the largest position): a model's positions are past .. past + q_len - 1
+    n_pos = max(past + q_len, W + 1, 2)
     cos, sin = rope_tables(D, n_pos, rope_base, query_states.dtype, query_states.device)
     kwargs = {"cos": cos, "sin": sin}
     if past == 0 and q_len > W:

@@ -280,8 +280,10 @@ class VectorQuantizedReRoPECache:
         self.sphere = sphere
         self.attention_mode = attention_mode
         self.generation_exact_window = generation_exact_window
-        self.key_codes = []      # per layer: codeword ids of the prefill, [B,H,N,1] uint8 (int16 above 256 codewords)
-        self.value_cache = []    # per layer: the prefill's values [B,H,N,D]
+        # per layer: codeword ids of the prefill, [B,H,N,1] uint8 (int16 above 256 codewords) -- 1 or 2 bytes per key
+        # next to the 2 D bytes of a value row, kept as the record of how the prefill was encoded.  The values (and
+        # keys) themselves are NOT kept: the generation steps run on the count state, O(C D) per (batch, head).
+        self.key_codes = []
         self.decode_state = []   # per layer: CountState or GenerationWindow
         self.seq_lengths = []    # per layer: tokens seen
         self.seen_tokens = 0
@@ -371,11 +373,16 @@ def apply_rope(x, cos, sin, positions, also_fixed=None):
     return out, x * cos[also_fixed] + rotate_half(x) * sin[also_fixed]
 
 
-def rerope_operands(query_states, key_states, position_ids, window_length, rope_base=10000.0):
+def rerope_operands(query_states, key_states, position_ids, window_length, rope_base=10000.0, past_length=0):
     """(q1, k1, q2) of ops/attn_vq.py:402-407: rotary at the true positions, and the query at the clamped position
-    window_length + 1.  position_ids [B,N]; states [B,H,N,D]."""
+    window_length + 1.  position_ids [B,N]; states [B,H,N,D].
+
+    The rotary tables are sized on the host, from `past_length + N` (the positions a model hands over are
+    past_length .. past_length + N - 1, or smaller with left padding): reading the largest position back from the
+    device would stall every layer's prefill on a device-to-host copy and keep the route out of a HIP graph.  A
+    position beyond the tables is clamped to their last row by the rotary kernel."""
     B, H, N, D = query_states.shape
-    n_pos = max(int(position_ids.max()) + 1, window_length + 2)
+    n_pos = max(past_length + N, window_length + 2)
     cos, sin = rope_tables(D, n_pos, rope_base, query_states.dtype, query_states.device)
     q1, q2 = apply_rope(query_states, cos, sin, position_ids, also_fixed=window_length + 1)
     k1 = apply_rope(key_states, cos, sin, position_ids)
@@ -472,10 +479,11 @@ def long_prefilling_per_key(query_states, key_states, value_states, position_ids
 
 def _remember(cache, layer_idx, ids, value_states, n_tokens, k1, key_states):
     """Record a prefill in the cache (what `update_prefill` keeps, ops/attn_vq.py:89-127): the sequence length, so
-    that the next seqlen_q == 1 call is recognised as a generation step; the codeword ids and values as given; and the
-    state the generation steps run on -- the count state over all keys, or, with `generation_exact_window`, the count
-    state below the far boundary of the next query plus the buffers of the exact keys above it.  The state itself is
-    built by the first generation step, from the tensors recorded here."""
+    that the next seqlen_q == 1 call is recognised as a generation step; the codeword ids; and the state the
+    generation steps run on -- the count state over all keys, or, with `generation_exact_window`, the count state
+    below the far boundary of the next query plus buffers of window + 256 exact keys above it.  The state is built
+    here (a fraction of a millisecond per layer) and nothing of the prefill's [B,H,N,D] tensors is referenced
+    afterwards: the memory of the cache is O(C D + window D) per (batch, head) plus the code bytes, whatever N is."""
     from .count_state import CountState, GenerationWindow
 
     if layer_idx == 0:
@@ -485,15 +493,12 @@ def _remember(cache, layer_idx, ids, value_states, n_tokens, k1, key_states):
         C = cache.codebook.shape[1]
         code_dtype = torch.uint8 if C <= 256 else torch.int16
         cache.key_codes.append(ids.to(code_dtype).unsqueeze(-1).contiguous())
-        cache.value_cache.append(value_states)
-
-        def build():  # run by the first generation step: a prefill that is never continued does not pay for it
-            state = CountState(B, H, C, D, value_states.device)
-            if cache.generation_exact_window:
-                return GenerationWindow(cache.window_length, k1, key_states, value_states, ids, n_tokens, state)
-            return state.add(ids, value_states)
-
-        cache.decode_state.append(build)
+        state = CountState(B, H, C, D, value_states.device)
+        if cache.generation_exact_window:
+            state = GenerationWindow(cache.window_length, k1, key_states, value_states, ids, n_tokens, state)
+        else:
+            state.add(ids, value_states)
+        cache.decode_state.append(state)
         cache.seq_lengths.append(n_tokens)
 
 
@@ -558,16 +563,15 @@ def dispatch_attn(query_states, key_states, value_states, position_ids, cache, l
     W = cache.window_length
     t = cache.seq_lengths[layer_idx]  # position of the new token
     ids = quantize_ids(key_states, cache.codebook)
-    if callable(cache.decode_state[layer_idx]):
-        cache.decode_state[layer_idx] = cache.decode_state[layer_idx]()
     state = cache.decode_state[layer_idx]
     scale = 1 / math.sqrt(D)
     cos, sin = rope_tables(D, max(W + 2, t + 1) if cache.generation_exact_window else W + 2, rope_base,
                            query_states.dtype, query_states.device)
     q2 = apply_rope(query_states, cos, sin, W + 1)
     if cache.generation_exact_window:
-        q1 = apply_rope(query_states, cos, sin, t)
-        k1 = apply_rope(key_states, cos, sin, t)
+        # true-position rotary at the positions the caller gives (per batch row; normally all equal to t)
+        q1 = apply_rope(query_states, cos, sin, position_ids)
+        k1 = apply_rope(key_states, cos, sin, position_ids)
         state.append(k1, key_states, value_states, ids)
         out = state.attend(q1, q2, cache.codebook, scale)
     else:
