@@ -466,10 +466,12 @@ def test_vq_prefill_pipelined_refuses_other_configurations():
 
 
 @pytest.mark.parametrize("with_rerope", [False, True])
-@pytest.mark.parametrize("B,H,N,D,K,W", [(1, 2, 1024, 128, 256, 256), (2, 2, 900, 64, 128, 128), (1, 1, 700, 128, 200, 384)])
+@pytest.mark.parametrize("B,H,N,D,K,W", [(1, 2, 1024, 128, 256, 256), (2, 2, 900, 64, 128, 128), (1, 1, 700, 128, 200, 384),
+                                          (1, 2, 650, 128, 256, 0), (2, 1, 333, 64, 128, 0)])
 def test_single_codebook_prefill_takes_the_codeword_route(B, H, N, D, K, W, with_rerope):
     """M = 1 with the block boundary: `attn_vq_prefill` runs the window kernel + count-weighted codeword kernel (far
-    context in O(N*K)); same oracle, and the per-key kernel forced on the same inputs agrees."""
+    context in O(N*K)); same oracle, and the per-key kernel forced on the same inputs agrees.  Includes lengths that
+    are no multiple of 128 and a window of 0 (only the keys of the query's own 128-block are exact)."""
     _say(f"single-codebook prefill B{B} H{H} N{N} D{D} K{K} W{W} rerope={with_rerope}")
     q, k, v, q2, k2 = (_randn(B, H, N, D, seed=110 + s) for s in range(5))
     cb = _randn(H, 1, K, D, seed=115, std=0.5)
