@@ -453,6 +453,19 @@ struct Pipe {
         });
     }
 
+    // Waits out the last P.V MFMAs with the O tuples as operands: whatever reads O afterwards -- the stores below, but
+    // also a copy the register allocator decides to make -- depends on this statement and cannot precede it.  (A
+    // compiler-made v_accvgpr_read right behind the last MFMA returned a stale last element of each tuple.)
+    static __device__ __forceinline__ void settle_o(Wave<Tag, D>& w) {
+        static_assert(DB == 4 || DB == 2, "head dims 128 and 64");
+        if constexpr (DB == 4)
+            asm volatile("s_nop 15"
+                         : "+a"(w.o[0][0]), "+a"(w.o[0][1]), "+a"(w.o[0][2]), "+a"(w.o[0][3]), "+a"(w.o[1][0]),
+                           "+a"(w.o[1][1]), "+a"(w.o[1][2]), "+a"(w.o[1][3])::"memory");
+        else
+            asm volatile("s_nop 15" : "+a"(w.o[0][0]), "+a"(w.o[0][1]), "+a"(w.o[1][0]), "+a"(w.o[1][1])::"memory");
+    }
+
     // Moves the reference maxima of the wave's rows for the tile whose scores are in `sc` (relative to the present
     // maxima, as the matrix pipe delivered them) and whose per-lane maxima are in mx.  Lazy rule: a row moves only when
     // the tile exceeds its maximum by more than 2^kLazy (or is the first one it sees).  Where a row moved, l and O are
@@ -464,7 +477,7 @@ struct Pipe {
         const bool any0 = mx[0] > ((w.m[0] == -INFINITY) ? -INFINITY : kLazy);
         const bool any1 = mx[1] > ((w.m[1] == -INFINITY) ? -INFINITY : kLazy);
         if (__builtin_amdgcn_ballot_w64(any0 || any1) == 0) return;
-        mfma_settle();  // O was last written by the previous tile's final MFMAs
+        settle_o(w);  // O was last written by the previous tile's final MFMAs
 #pragma unroll
         for (int qb = 0; qb < 2; ++qb) {
             const float rel = join_halves_max(mx[qb]);
@@ -515,6 +528,35 @@ struct Pipe {
         });
     }
 
+    // The same without a staging area: every lane stores the 8-byte pieces of its own row (64 rows per instruction).
+    // For callers whose LDS is in use when the rows are ready (tiles of the next query tile already on their way).
+    static __device__ __forceinline__ void store_direct(Wave<Tag, D>& w, uint16_t* out_base, int64_t sn,
+                                                        float* lse, int row0, int n_rows, int lane) {
+        const int n = lane & 31, half = lane >> 5;
+        settle_o(w);
+#pragma unroll
+        for (int qb = 0; qb < 2; ++qb) {
+            const float l_tot = join_halves_sum(w.l[qb][0] + w.l[qb][1]);
+            const int row = row0 + qb * 32 + n;
+            if (row >= n_rows) continue;
+            const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+            uint16_t* dst = out_base + (int64_t)row * sn;
+#pragma unroll
+            for (int db = 0; db < DB; ++db) {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    uint2 pk;
+                    pk.x = (uint32_t)Elem<Tag>::to_bits(w.o[qb][db][4 * g] * inv) |
+                           ((uint32_t)Elem<Tag>::to_bits(w.o[qb][db][4 * g + 1] * inv) << 16);
+                    pk.y = (uint32_t)Elem<Tag>::to_bits(w.o[qb][db][4 * g + 2] * inv) |
+                           ((uint32_t)Elem<Tag>::to_bits(w.o[qb][db][4 * g + 3] * inv) << 16);
+                    *reinterpret_cast<uint2*>(dst + db * 32 + 8 * g + 4 * half) = pk;
+                }
+            }
+            if (lse != nullptr && half == 0) lse[row] = l_tot > 0.f ? w.m[qb] + fast_log2(l_tot) : -INFINITY;
+        }
+    }
+
     // Normalise and store the wave's 64 output rows; lse2 = m + log2(l).  A row that saw no key stores 0 / -inf.
     // In the accumulator layout a lane holds 4-element pieces of ONE row: stored directly, every instruction would
     // touch 64 rows.  The rows go through the wave's own LDS staging area instead (kStoreBytes at lds_stage, rows
@@ -522,14 +564,12 @@ struct Pipe {
     // rows, 16 bytes per lane.  The caller makes sure no wave still reads what lies in that LDS area.
     static constexpr int kStoreRowBytes = G::kRowBytes + 8;
     static constexpr int kStoreBytes = kWaveRows * kStoreRowBytes;
-    static __device__ __forceinline__ void store(const Wave<Tag, D>& w, uint16_t* out_base, int64_t sn, float* lse,
+    static __device__ __forceinline__ void store(Wave<Tag, D>& w, uint16_t* out_base, int64_t sn, float* lse,
                                                  int row0, int n_rows, int lane, char* lds_stage) {
         const int n = lane & 31, half = lane >> 5;
-        mfma_settle();
+        settle_o(w);
 #pragma unroll
         for (int qb = 0; qb < 2; ++qb) {
-#pragma unroll
-            for (int db = 0; db < DB; ++db) asm volatile("" : "+a"(const_cast<f32x16_t&>(w.o[qb][db])));  // read after the wait
             const float l_tot = join_halves_sum(w.l[qb][0] + w.l[qb][1]);
             const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
             char* dst = lds_stage + (qb * 32 + n) * kStoreRowBytes;

@@ -18,6 +18,7 @@
 // tiles per query tile the workgroup brings both K sources and each wave reads the one it needs; no per-element
 // selection exists elsewhere, masks only on the causal diagonal, at the lower window edge and at the end of the
 // sequence.  The tile schedule is plain arithmetic on (m0, W, N).
+#include <algorithm>
 #include <mutex>
 
 #include "vqa_flash2.h"
@@ -43,6 +44,7 @@ struct Params {
     int causal, all_far;  // kVq
     int strict;           // kWindow: j >= i - W instead of the block rule
     int pair_tiles;
+    int tiles_per_wg;  // sliding-window kinds: query tiles one workgroup walks
     float scale_log2e;
 };
 
@@ -309,10 +311,286 @@ __global__ __launch_bounds__(64 * waves_of<KIND>(), 1) void prefill_pipe_kernel(
     }
 
     // the output rows leave through LDS (every wave its own part of the tile buffers) once no wave reads tiles any more
+    Pipe::settle_o(w);
     __syncthreads();
     static_assert((size_t)NW * Pipe::kStoreBytes <= lds_bytes<D, KIND>(), "staging area exceeds the tile buffers");
     Pipe::store(w, p.out + b * p.o_sb + h * p.o_sh, p.o_sn, p.lse ? p.lse + (int64_t)bh * p.N : nullptr, row0, p.N,
                 lane, smem + wave * Pipe::kStoreBytes);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// Sliding-window kinds (kWindow, kRerope): 128-row query tiles (2 waves), two workgroups per CU, and every workgroup
+// walks a run of consecutive query tiles of one (batch, head).  A query tile meets only (W + 128) / 64 key tiles, so
+// what surrounds its key loop weighs as much as the loop: a cold start (first tiles and queries from HBM), the
+// drained software pipeline, the output rows, the launch of the next workgroup.  Walking a run removes the launches
+// and lets the LAST iteration of a query tile -- which has no next key tile to score -- bring the first tiles and the
+// queries of the next query tile instead, under its exponentials and its P.V product.
+//
+// Tile buffers: first-source K [2] | V [2] | (kRerope) second-source K [1].  Their parity is logical: a query tile may
+// end on either one, the next starts on the free V buffer (`flip`).  The sequence length is a multiple of 64 (the
+// host sends other lengths to the general kernel), so every tile copy is a whole tile.
+// ---------------------------------------------------------------------------------------------------------------
+template <int KIND>
+constexpr size_t window_lds_bytes(int tile_bytes) {
+    return (size_t)tile_bytes * (KIND == kRerope ? 5 : 4);
+}
+
+template <typename Tag, int D, int KIND>
+__global__ __launch_bounds__(128, 1) void window_pipe_kernel(Params p) {
+    static_assert(KIND == kWindow || KIND == kRerope, "sliding-window kinds only");
+    typedef Geom<D> G;
+    constexpr int NW = 2;
+    constexpr int kBM = NW * flash2::kWaveRows;
+    typedef flash2::Pipe<Tag, D, NW> Pipe;
+    typedef typename Pipe::KDma KDma;
+    typedef typename Pipe::VDma VDma;
+    extern __shared__ __attribute__((aligned(1024))) char smem[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t lds0 = flash::lds_addr_of(smem);
+    auto lds_ptr = [&](uint32_t addr) { return smem + (addr - lds0); };
+
+    // every XCD (own L2) gets whole (batch, head) problems
+    int bh, slot;
+    {
+        const int n_slots = gridDim.x, n_bh = gridDim.y;
+        const int id = blockIdx.x + n_slots * blockIdx.y;
+        if (n_bh % 8 == 0) {
+            const int xcd = id & 7, k = id >> 3;
+            bh = xcd + 8 * (k / n_slots);
+            slot = k % n_slots;
+        } else {
+            bh = blockIdx.y;
+            slot = blockIdx.x;
+        }
+    }
+    const int b = bh / p.H, h = bh % p.H;
+    const int n_tiles = (p.N + kBM - 1) / kBM;
+    // The workgroups of a (batch, head) take its query tiles in turn (workgroup s: tiles s, s + S, s + 2S, ...), so
+    // the workgroups running at one time work on neighbouring query tiles and share their K / V tiles in the L2.
+    // (Runs of ADJACENT tiles per workgroup were measured 1.2 x slower: every workgroup then streams a region of
+    // its own and nothing is shared.)
+    const int t_step = gridDim.x;
+    const int t_begin = slot, t_end = n_tiles;
+    if (t_begin >= t_end) return;  // (workgroup-uniform)
+
+    const uint16_t* ka = p.ka.p + b * p.ka.sb + h * p.ka.sh;
+    const uint16_t* kc = p.kc.p + b * p.kc.sb + h * p.kc.sh;
+    const uint16_t* v_src = p.v.p + b * p.v.sb + h * p.v.sh;
+    const uint16_t* q_src = p.q.p + b * p.q.sb + h * p.q.sh;
+    const uint16_t* q2_src = p.q2.p + b * p.q2.sb + h * p.q2.sh;
+    uint16_t* out = p.out + b * p.o_sb + h * p.o_sh;
+    float* lse = p.lse ? p.lse + (int64_t)bh * p.N : nullptr;
+
+    KDma kd_a;
+    VDma vd;
+    kd_a.init(wave, lane, p.ka.sn);
+    vd.init(wave, lane, p.v.sn);
+    const int64_t ka_step = (int64_t)kBN * p.ka.sn * 2, v_step = (int64_t)kBN * p.v.sn * 2;
+    const int n_key_tiles = p.N / kBN;  // all whole
+    auto copy_tile = [&](uint32_t lds_tile, const uint16_t* base, int64_t sn, int n0, auto is_v)
+        __attribute__((always_inline)) {
+        flash::TileCopy<D, decltype(is_v)::value, NW> c;
+        c.init(wave, flash2::opaque_lane(lane));
+        c.load_full(lds_ptr(lds_tile), base, sn, n0);
+    };
+
+    // geometry of one query tile for this wave
+    struct Tile {
+        int m0, row0, edge_w, lo_w, u0, n_iter;
+    };
+    auto tile_of = [&](int t) {
+        Tile g;
+        g.m0 = t * kBM;
+        g.row0 = g.m0 + wave * flash2::kWaveRows;
+        // kRerope: the second pair scores the keys j < i - W: whole tiles below edge_w, half of the tile at edge_w
+        g.edge_w = KIND == kRerope ? g.row0 - p.window : -1;
+        // lowest visible key of the wave's rows (of its first row for the strict rule)
+        g.lo_w = p.strict ? g.row0 - p.window : (g.row0 / kBlock) * kBlock - p.window;
+        g.u0 = max(0, g.m0 - p.window) / kBN;
+        g.n_iter = (min(p.N, g.m0 + kBM) + kBN - 1) / kBN;
+        return g;
+    };
+    Tile g = tile_of(t_begin);
+    int flip = 0;  // physical buffer of logical parity 0
+    auto s_ka = [&](int par) { return lds0 + (uint32_t)(((par ^ flip) & 1) * G::kTileBytes); };
+    auto s_v = [&](int par) { return lds0 + (uint32_t)((2 + ((par ^ flip) & 1)) * G::kTileBytes); };
+    const uint32_t s_kc = lds0 + 4u * G::kTileBytes;
+    // second-source tiles: up to the last wave's edge tile
+    auto needs_c = [&](const Tile& x, int u) { return KIND == kRerope && u * kBN <= x.m0 + (NW - 1) * flash2::kWaveRows - p.window; };
+    auto wave_reads_c = [&](int u) { return KIND == kRerope && u * kBN <= g.edge_w; };
+    auto k_tile_of_wave = [&](int u, int par) { return wave_reads_c(u) ? s_kc : s_ka(par); };
+    // first tiles of a query tile (as a block): K(u0), V(u0), K(u0 + 1), and the second source of K(u0)
+    auto request_first = [&](const Tile& x) __attribute__((always_inline)) {
+        copy_tile(s_ka(0), ka, p.ka.sn, x.u0 * kBN, std::false_type{});
+        copy_tile(s_v(0), v_src, p.v.sn, x.u0 * kBN, std::true_type{});
+        if (x.u0 + 1 < x.n_iter) copy_tile(s_ka(1), ka, p.ka.sn, (x.u0 + 1) * kBN, std::false_type{});
+        if (needs_c(x, x.u0)) copy_tile(s_kc, kc, p.kc.sn, x.u0 * kBN, std::false_type{});
+    };
+    // a wave that meets second-pair keys starts with the second query and changes over at its edge tile
+    auto first_query_of = [&](const Tile& x, const uint16_t*& src, int64_t& sn_q) {
+        const bool second = KIND == kRerope && x.edge_w >= 0;
+        src = second ? q2_src : q_src;
+        sn_q = second ? p.q2.sn : p.q.sn;
+    };
+
+    flash2::Wave<Tag, D> w;
+    Scores s_even, s_odd;
+    typename Pipe::Frags kf, vf;
+    float mx[2];
+    const typename Pipe::TileRequest no_req{nullptr, 0};
+
+    request_first(g);
+    {
+        const uint16_t* src;
+        int64_t sn_q;
+        first_query_of(g, src, sn_q);
+        flash::load_q<Tag, D>(w.q[0], src, sn_q, g.row0, p.N, lane);
+        flash::load_q<Tag, D>(w.q[1], src, sn_q, g.row0 + 32, p.N, lane);
+        flash2::prescale_q<Tag, D>(w.q[0], p.scale_log2e);
+        flash2::prescale_q<Tag, D>(w.q[1], p.scale_log2e);
+    }
+
+    for (int t = t_begin; t < t_end; t += t_step) {
+    w.init();
+    mx[0] = mx[1] = -INFINITY;
+    const int row0 = g.row0;
+
+    // masks of tile u for this wave: causal diagonal, lower window edge, tiles past the wave's last row
+    auto mask_tile = [&](Scores& sn, int u) __attribute__((always_inline)) {
+        const int n0 = u * kBN;
+        const int lo_last = g.lo_w + (p.strict ? flash2::kWaveRows - 1 : 0);  // of the wave's last row
+        const bool whole = n0 + kBN - 1 <= row0 && u < g.n_iter && n0 >= lo_last;
+        if (whole) return;  // (wave-uniform)
+        flash2::mfma_settle(sn);  // the scores below were produced by the last MFMAs
+        const int lane_o = flash2::opaque_lane(lane);  // keeps the predicates inside this branch
+        const int half = lane_o >> 5;
+        const int j_hi = u < g.n_iter ? p.N : 0;  // no such tile: nothing visible
+#pragma unroll
+        for (int qb = 0; qb < 2; ++qb) {
+            const int i = row0 + qb * 32 + (lane_o & 31);
+            const int lim = min(j_hi, i + 1);  // keys lo <= j < lim are visible
+            const int lo = g.lo_w + (p.strict ? i - row0 : 0);
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int j = n0 + kb * 32 + flash::key_of_reg(r, half);
+                    sn.s[qb][kb][r] = (j < lim && j >= lo) ? sn.s[qb][kb][r] : -INFINITY;
+                }
+        }
+    };
+    // after the scores of tile u: masks, and at the wave's ReRoPE edge tile the change-over to the first pair (the
+    // scores so far are q2.k2; keys with i - j <= W take q1.k1, and q1 serves every later tile)
+    auto finish_scores = [&](Scores& sn, int u, int par) __attribute__((always_inline)) {
+        mask_tile(sn, u);
+        if constexpr (KIND == kRerope) {
+            if (u * kBN == g.edge_w) {  // (wave-uniform; every key of this tile is visible to every row of the wave)
+                flash::load_q<Tag, D>(w.q[0], q_src, p.q.sn, row0, p.N, lane);
+                flash::load_q<Tag, D>(w.q[1], q_src, p.q.sn, row0 + 32, p.N, lane);
+                flash2::prescale_q<Tag, D>(w.q[0], p.scale_log2e);
+                flash2::prescale_q<Tag, D>(w.q[1], p.scale_log2e);
+                const int lane_o = flash2::opaque_lane(lane);
+                const int half = lane_o >> 5, n = lane_o & 31;
+                Pipe::second_pair(w, sn, s_ka(par), lane, [&](int qb, int kb, int r) {
+                    // i - j <= W  with  i = row0 + qb*32 + n,  j = edge_w + kb*32 + key:  qb*32 + n <= kb*32 + key
+                    return qb * 32 + n <= kb * 32 + flash::key_of_reg(r, half);
+                });
+            }
+        }
+    };
+
+    // first tile: scores, masks, row maxima (nothing to overlap with yet)
+    flash::wait_tile_loads();
+    __syncthreads();
+    Pipe::k_head(kf, k_tile_of_wave(g.u0, 0), lane);
+    Pipe::template score_phase<true, false, false, false>(w, s_even, kf, s_odd, vf, 0u, lane, kd_a, no_req, vd, no_req);
+    finish_scores(s_even, g.u0, 0);
+    Pipe::template pv_phase<false, true>(w, vf, s_odd, s_even, mx);
+
+    // rows of this wave's share of K tile u + 2 and V tile u + 1
+    const int r2 = (g.u0 + 2) * kBN + wave * KDma::kRowsPerWave;
+    const char* ka_rows = reinterpret_cast<const char*>(ka + (int64_t)r2 * p.ka.sn);
+    const char* v_rows = reinterpret_cast<const char*>(v_src + (int64_t)(r2 - kBN) * p.v.sn);
+    // Iteration u finishes tile u (exponentials, P.V) and prepares tile u + 1 (scores, masks, row maxima); K(u+1) and
+    // V(u) were requested one iteration earlier and sit in the buffers of parity u + 1 and u.  It requests K(u+2) and
+    // V(u+1), which ride on the score MFMAs.
+    auto iteration = [&](auto u_is_odd, int u) __attribute__((always_inline)) {
+        constexpr int par = decltype(u_is_odd)::value ? 1 : 0;
+        Scores& sc = par ? s_odd : s_even;
+        Scores& sn = par ? s_even : s_odd;
+        flash::wait_tile_loads();
+        __syncthreads();  // K(u+1) and V(u) are complete; every wave is done with K(u) and V(u-1)
+        if constexpr (KIND == kRerope) {
+            // the one second-source buffer is free now: the tile about to be scored is brought and waited for (once per
+            // query tile; the other workgroup of the CU computes meanwhile)
+            if (needs_c(g, u + 1)) {  // (workgroup-uniform)
+                copy_tile(s_kc, kc, p.kc.sn, (u + 1) * kBN, std::false_type{});
+                flash::wait_tile_loads();
+                __syncthreads();
+            }
+        }
+        Pipe::k_head(kf, k_tile_of_wave(u + 1, par + 1), lane);
+        typename Pipe::TileRequest kr, vr;
+        // K(u+2) may lie past the sequence for the last query tile: the copy then repeats the last tile into a buffer
+        // nobody reads any more
+        kr.rows = (u + 2 < n_key_tiles) ? ka_rows : ka_rows - ka_step;
+        kr.lds = KDma::lds_of_wave(s_ka(par), wave);
+        vr.rows = v_rows;
+        vr.lds = VDma::lds_of_wave(s_v(par + 1), wave);
+        ka_rows += ka_step, v_rows += v_step;
+        Pipe::update_max(w, mx, sc);
+        Pipe::template score_phase<true, true, true, true>(w, sn, kf, sc, vf, s_v(par), lane, kd_a, kr, vd, vr);
+        finish_scores(sn, u + 1, par + 1);
+        mx[0] = mx[1] = -INFINITY;
+        Pipe::template pv_phase<true, true>(w, vf, sc, sn, mx);
+    };
+    // The last iteration finishes the last tile.  There is no next key tile; in its place the first tiles of the next
+    // query tile are requested (both K buffers and the other V buffer are free) and its queries are loaded, and both
+    // are on their way while the exponentials and the P.V product run and the output rows leave.
+    const bool has_next = t + t_step < t_end;
+    const Tile gn = tile_of(has_next ? t + t_step : t);
+    // (one body: a query tile that ends on the odd buffer moves its last scores over first, 64 moves per query tile)
+    auto last_iteration = [&](int par) __attribute__((always_inline)) {
+        Scores& sc = s_even;
+        Scores& sn = s_odd;  // (unused: no scores are produced)
+        flash::wait_tile_loads();
+        __syncthreads();  // V(u) is complete; every wave is done with K(u) and V(u-1)
+        const uint32_t lds_v_now = s_v(par);
+        if (has_next) {  // (the query fragments are free: this iteration scores nothing)
+            flip ^= par ^ 1;  // logical parity 0 of the next query tile = the V buffer that is free now
+            request_first(gn);
+            const uint16_t* src;
+            int64_t sn_q;
+            first_query_of(gn, src, sn_q);
+            flash::load_q<Tag, D>(w.q[0], src, sn_q, gn.row0, p.N, lane);
+            flash::load_q<Tag, D>(w.q[1], src, sn_q, gn.row0 + 32, p.N, lane);
+        }
+        Pipe::update_max(w, mx, sc);
+        Pipe::template score_phase<false, true, true, false>(w, sn, kf, sc, vf, lds_v_now, lane, kd_a, no_req, vd, no_req);
+        Pipe::template pv_phase<true, false>(w, vf, sc, sn, mx);
+        Pipe::settle_o(w);  // (here, not only in the store: nothing may touch O between the last MFMA and the wait)
+    };
+    int u = g.u0;
+    for (; u + 2 < g.n_iter; u += 2) {
+        iteration(std::false_type{}, u);
+        iteration(std::true_type{}, u + 1);
+    }
+    int last_par = 0;
+    if (u + 1 < g.n_iter) {
+        iteration(std::false_type{}, u);
+        s_even = s_odd;
+        last_par = 1;
+    }
+    last_iteration(last_par);
+    Pipe::store_direct(w, out, p.o_sn, lse, row0, p.N, lane);
+    if (has_next) {
+        flash2::prescale_q<Tag, D>(w.q[0], p.scale_log2e);
+        flash2::prescale_q<Tag, D>(w.q[1], p.scale_log2e);
+    }
+    g = gn;
     }
 }
 
@@ -345,10 +623,44 @@ int launch(Params p, int B, hipStream_t stream) {
     return launch_status();
 }
 
+template <typename Tag, int D, int KIND>
+int launch_window(Params p, int B, hipStream_t stream) {
+    constexpr size_t kLds = window_lds_bytes<KIND>(Geom<D>::kTileBytes);
+    static std::mutex mu;
+    static bool raised[kMaxDevices] = {};
+    int dev = 0;
+    const int rc = device_of_pointer(p.q.p, &dev);
+    if (rc != VQA_OK) return rc;
+    {
+        std::lock_guard<std::mutex> lock(mu);
+        if (!raised[dev]) {
+            if (hipFuncSetAttribute(reinterpret_cast<const void*>(&window_pipe_kernel<Tag, D, KIND>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLds) != hipSuccess) {
+                (void)hipGetLastError();
+                return VQA_ERR_LAUNCH_FAILED;
+            }
+            raised[dev] = true;
+        }
+    }
+    // runs of consecutive query tiles per workgroup: as long as possible while two rounds of workgroups remain for
+    // the 512 places (256 CUs x 2) of the chip
+    const int n_tiles = (p.N + 127) / 128;
+    const int64_t total = (int64_t)n_tiles * B * p.H;
+    p.tiles_per_wg = (int)std::max<int64_t>(1, std::min<int64_t>(16, total / 1024));
+    const dim3 grid((n_tiles + p.tiles_per_wg - 1) / p.tiles_per_wg, B * p.H);
+    hipLaunchKernelGGL((window_pipe_kernel<Tag, D, KIND>), grid, dim3(128), kLds, stream, p);
+    return launch_status();
+}
+
 template <typename Tag, int KIND>
 int launch_d(const Params& p, int B, int D, hipStream_t stream) {
-    if (D == 64) return launch<Tag, 64, KIND>(p, B, stream);
-    if (D == 128) return launch<Tag, 128, KIND>(p, B, stream);
+    if constexpr (KIND == kVq) {
+        if (D == 64) return launch<Tag, 64, KIND>(p, B, stream);
+        if (D == 128) return launch<Tag, 128, KIND>(p, B, stream);
+    } else {
+        if (D == 64) return launch_window<Tag, 64, KIND>(p, B, stream);
+        if (D == 128) return launch_window<Tag, 128, KIND>(p, B, stream);
+    }
     return VQA_ERR_UNSUPPORTED_HEAD_DIM;
 }
 
@@ -365,7 +677,9 @@ bool prefill_pipe_applies(int window, int boundary_is_block, bool has_exact, boo
 }
 
 // sliding-window kinds: window_rule 0 = strict (j >= i - W), 1 = block rule, 2 = block rule with the ReRoPE pair
-bool window_pipe_applies(int window, int N) { return window > 0 && window % pipe::kBlock == 0 && window < N; }
+bool window_pipe_applies(int window, int N) {
+    return window > 0 && window % pipe::kBlock == 0 && window < N && N % pipe::kBN == 0;
+}
 
 template <typename Tag>
 int prefill_pipe_run(const View& q, const View& ka, const View& kc, const View& v, uint16_t* out, int64_t o_sb,
@@ -381,6 +695,7 @@ int prefill_pipe_run(const View& q, const View& ka, const View& kc, const View& 
     p.all_far = all_far ? 1 : 0;
     p.strict = 0;
     p.pair_tiles = 0;
+    p.tiles_per_wg = 1;
     p.scale_log2e = scale_log2e;
     return pipe::launch_d<Tag, pipe::kVq>(p, B, D, stream);
 }
@@ -399,6 +714,7 @@ int window_pipe_run(const View& q1, const View& q2, const View& k1, const View& 
     p.all_far = 0;
     p.strict = window_rule == 0 ? 1 : 0;
     p.pair_tiles = 0;
+    p.tiles_per_wg = 1;
     p.scale_log2e = scale_log2e;
     if (window_rule == 2) return pipe::launch_d<Tag, pipe::kRerope>(p, B, D, stream);
     return pipe::launch_d<Tag, pipe::kWindow>(p, B, D, stream);

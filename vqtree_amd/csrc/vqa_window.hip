@@ -537,8 +537,8 @@ int local_attn(const void* q1, const void* q2, const void* k1, const void* k2, c
     // rows) are not overlapped with anything on its SIMDs, so it needs long windows: measured over batch x heads
     // 8 - 128, 2k - 32k tokens, windows 128 - 2048 it takes 0.77 - 0.99 of the tiled kernel's time from W = 1024 on
     // with at least 2048 workgroups, 1.03 - 1.47 below.
-    if (mode <= kLocalRerope && window_pipe_applies(window, N) && (D == 64 || D == 128) && window >= 1024 &&
-        (int64_t)((N + 127) / 128) * B * H >= 2048) {
+    if (mode <= kLocalRerope && window_pipe_applies(window, N) && (D == 64 || D == 128) && window >= 128 &&
+        (int64_t)((N + 127) / 128) * B * H >= 1) {
         const int rc = validate(p, B, D);
         if (rc != VQA_OK) return rc;
         return window_pipe_run<Tag>(p.qa, p.qb, p.ka, p.kb, p.v, p.out, p.o_sb, p.o_sh, p.o_sn, p.lse, B, H, N, D,
