@@ -76,11 +76,14 @@ def test_window_modes(mode, B, H, N, D, W):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("mode", ["strict", "loose", "rerope"])
-@pytest.mark.parametrize("N,D,W", [(4096, 128, 1024), (4000, 128, 1152), (4096, 64, 2048)])
+@pytest.mark.parametrize("N,D,W", [(4096, 128, 1024), (4032, 128, 1152), (4096, 64, 2048), (4096, 128, 512),
+                                   (4000, 128, 1152)])
 def test_window_modes_on_the_pipelined_core(mode, N, D, W, dtype):
-    """64 (batch, head) units x >= 4000 tokens with a window of >= 1024 keys that is a multiple of 128: here
-    vqa_local_attn_* runs the sliding-window kinds of the pipelined core (128-row workgroups; for ReRoPE the second
-    pair through a change of the query operand at each wave's window-edge tile).  Three units against the oracle."""
+    """64 (batch, head) units x ~4000 tokens with a window of >= 512 keys that is a multiple of 128 and a length that
+    is a multiple of 64: here vqa_local_attn_* runs the sliding-window kinds of the pipelined core (128-row workgroups
+    that walk several query tiles each; for ReRoPE the second pair through a change of the query operand at each
+    wave's window-edge tile).  N = 4000 is the same call on the general kernel (length not a multiple of 64).  Three
+    units against the oracle."""
     _say(f"window on the pipelined core {mode} N{N} D{D} W{W} {dtype}")
     B, H = 2, 32
     g = torch.Generator(device="cuda").manual_seed(53)

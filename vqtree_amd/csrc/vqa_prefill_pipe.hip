@@ -3,11 +3,11 @@
 //   kVq      VQ prefill: far keys (j < boundary(i)) are scored against the reconstructed keys K_hat, recent keys against
 //            the exact keys, both with the same query tensor, boundary(i) = max(0, floor((i - W) / 128) * 128) with W a
 //            multiple of 128 -- the configuration of the reference's long prefill (ops/attn_vq.py:311, window lengths
-//            are multiples of its 128 block) -- or every key far (no exact keys).
+//            are multiples of its 128 block) -- or every key far (no exact keys).  prefill_pipe_kernel.
 //   kWindow  sliding window with one operand pair: keys j <= i with j >= i - W (strict) or j >= floor(i/128)*128 - W
-//            (the reference's block rule, ops/triton_fused_local_attn2.py), W a multiple of 128.
+//            (the reference's block rule, ops/triton_fused_local_attn2.py), W a multiple of 128.  window_pipe_kernel.
 //   kRerope  the block-rule window with the ReRoPE pair rule (ops/triton_fused_local_attn_rerope.py:38-78): score
-//            q1.k1 where i - j <= W, else q2.k2.
+//            q1.k1 where i - j <= W, else q2.k2.  window_pipe_kernel.
 //
 // Everything else (a second query / key pair next to quantised keys, the exact boundary rule, other window lengths)
 // stays with the general kernel in vqa_window.hip.
@@ -48,34 +48,18 @@ struct Params {
     float scale_log2e;
 };
 
-// Workgroup shapes.  kVq: 4 waves = 256 query rows, one workgroup per CU (long key loops; the tile copies serve 256
-// rows).  Window kinds: 2 waves = 128 query rows and TWO workgroups per CU: a query tile meets only (W + 128) / 64 key
-// tiles, so the start of a workgroup (first tiles and queries from a cold start) and its end (output rows) are a
-// large part of its life and must overlap with another workgroup's products; 128-row tiles also waste fewer
-// (wave, tile) blocks below the window (a wave idles while the waves of the other 128-row block still have keys).
-template <int KIND>
-constexpr int waves_of() {
-    return KIND == kVq ? 4 : 2;
-}
-// LDS: first-source K tiles [2] | V tiles [2] | second-source K tiles: [2] for kVq, [1] for kRerope (two workgroups
-// must fit the 160 KB: only the first two key tiles of a query tile have a second source, the second one is brought
-// when the first has been scored), none for kWindow
-template <int KIND>
-constexpr int second_source_slots() {
-    return KIND == kVq ? 2 : (KIND == kRerope ? 1 : 0);
-}
-template <int D, int KIND>
+// kVq: 4 waves = 256 query rows, one workgroup per CU (long key loops; the tile copies serve 256 rows).
+// LDS: exact-K tiles [2] | reconstructed-K tiles [2] | V tiles [2]
+constexpr int kBM = flash2::kBM;
+template <int D>
 constexpr size_t lds_bytes() {
-    return (size_t)Geom<D>::kTileBytes * (4 + second_source_slots<KIND>());
+    return (size_t)Geom<D>::kTileBytes * 6;
 }
 
-template <typename Tag, int D, int KIND>
-__global__ __launch_bounds__(64 * waves_of<KIND>(), 1) void prefill_pipe_kernel(Params p) {
+template <typename Tag, int D>
+__global__ __launch_bounds__(flash2::kThreads, 1) void prefill_pipe_kernel(Params p) {
     typedef Geom<D> G;
-    constexpr int NW = waves_of<KIND>();
-    constexpr int kBM = NW * flash2::kWaveRows;  // query rows per workgroup
-    constexpr int kSlotsC = second_source_slots<KIND>();
-    typedef flash2::Pipe<Tag, D, NW> Pipe;
+    typedef flash2::Pipe<Tag, D> Pipe;
     typedef typename Pipe::KDma KDma;
     typedef typename Pipe::VDma VDma;
     extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -85,8 +69,8 @@ __global__ __launch_bounds__(64 * waves_of<KIND>(), 1) void prefill_pipe_kernel(
     // tiles are named by their LDS byte address
     const uint32_t lds0 = flash::lds_addr_of(smem);
     auto s_ka = [&](int par) { return lds0 + (uint32_t)((par & 1) * G::kTileBytes); };
-    auto s_v = [&](int par) { return lds0 + (uint32_t)((2 + (par & 1)) * G::kTileBytes); };
-    auto s_kc = [&](int par) { return lds0 + (uint32_t)((4 + (kSlotsC == 2 ? (par & 1) : 0)) * G::kTileBytes); };
+    auto s_kc = [&](int par) { return lds0 + (uint32_t)((2 + (par & 1)) * G::kTileBytes); };
+    auto s_v = [&](int par) { return lds0 + (uint32_t)((4 + (par & 1)) * G::kTileBytes); };
     auto lds_ptr = [&](uint32_t addr) { return smem + (addr - lds0); };
 
     // every XCD (own L2) gets whole (batch, head) problems; late and early query tiles are paired per workgroup so
@@ -113,7 +97,6 @@ __global__ __launch_bounds__(64 * waves_of<KIND>(), 1) void prefill_pipe_kernel(
     const uint16_t* kc = p.kc.p + b * p.kc.sb + h * p.kc.sh;
     const uint16_t* v_src = p.v.p + b * p.v.sb + h * p.v.sh;
     const uint16_t* q_src = p.q.p + b * p.q.sb + h * p.q.sh;
-    const uint16_t* q2_src = p.q2.p + b * p.q2.sb + h * p.q2.sh;
 
     // whole-tile copies that ride on the score MFMAs: per-lane offsets once per kernel (one set per row stride)
     KDma kd_a, kd_c;
@@ -124,12 +107,12 @@ __global__ __launch_bounds__(64 * waves_of<KIND>(), 1) void prefill_pipe_kernel(
     // any other tile copy (first tiles of a pass, tiles that run over the end of the sequence, the second K source of
     // a boundary tile): issued as a block
     auto copy_k = [&](uint32_t lds_tile, const uint16_t* base, int64_t sn, int n0) __attribute__((always_inline)) {
-        flash::TileCopy<D, false, NW> c;
+        flash::TileCopy<D, false> c;
         c.init(wave, flash2::opaque_lane(lane));
         c.load(lds_ptr(lds_tile), base, sn, n0, p.N);
     };
     auto copy_v = [&](uint32_t lds_tile, int n0) __attribute__((always_inline)) {
-        flash::TileCopy<D, true, NW> c;
+        flash::TileCopy<D, true> c;
         c.init(wave, flash2::opaque_lane(lane));
         c.load(lds_ptr(lds_tile), v_src, p.v.sn, n0, p.N);
     };
@@ -141,63 +124,44 @@ __global__ __launch_bounds__(64 * waves_of<KIND>(), 1) void prefill_pipe_kernel(
     const int row0 = m0 + wave * flash2::kWaveRows;  // this wave's 64 rows (inside one 128-row block)
     if (pass) __syncthreads();  // the previous query tile's last reads of the LDS buffers are done
 
+    // first exact key of the two 128-row blocks of the workgroup, and of this wave's block
     const int kNever = 0x7fffffff;
-    // kVq: first exact key of the two 128-row blocks of the workgroup, and of this wave's block
-    const int fb_lo = (KIND != kVq || p.all_far) ? kNever : max(0, m0 - p.window);
-    const int fb_hi = (KIND != kVq || p.all_far) ? kNever : max(0, m0 + kBM - kBlock - p.window);
-    const int fb_w = (wave * flash2::kWaveRows < kBlock) ? fb_lo : fb_hi;
-    // kRerope: the second pair scores the keys j < i - W: whole tiles below edge_w, half of the tile at edge_w
-    const int edge_w = KIND == kRerope ? row0 - p.window : -1;
-    // window kinds: lowest visible key of the wave's rows (lo_w + row offset for the strict rule) and of the query tile
-    const int lo_w = KIND == kVq ? 0 : (p.strict ? row0 - p.window : (row0 / kBlock) * kBlock - p.window);
-    // tiles [u0, n_iter): from the query tile's lowest visible key up to its last row (causal) or all keys
-    const int u0 = KIND == kVq ? 0 : max(0, m0 - p.window) / kBN;
-    const int hi_key = (KIND != kVq || p.causal) ? min(p.N, m1 + 1) : p.N;
+    const int fb_lo = p.all_far ? kNever : max(0, m0 - p.window);
+    const int fb_hi = p.all_far ? kNever : max(0, m0 + kBlock - p.window);
+    const int fb_w = (wave < 2) ? fb_lo : fb_hi;
+    // tiles [0, n_iter): keys up to the last row of the query tile (causal) or all of them
+    const int hi_key = p.causal ? min(p.N, m1 + 1) : p.N;
     const int n_iter = (hi_key + kBN - 1) / kBN;
     const int n_whole = min(n_iter, p.N / kBN);  // tiles that lie inside the sequence with all 64 rows
     // K tiles a key tile needs (workgroup-uniform) and the buffer this wave scores from
-    auto needs_c = [&](int u) {
-        if (KIND == kVq) return u * kBN < fb_hi;
-        if (KIND == kRerope) return u * kBN <= m0 + (NW - 1) * flash2::kWaveRows - p.window;  // the last wave's edge tile
-        return false;
-    };
-    auto needs_a = [&](int u) { return KIND == kVq ? u * kBN >= fb_lo : true; };
-    // (a single second-source slot holds the tile being scored: the next one cannot be requested ahead, see iteration)
+    auto needs_far = [&](int u) { return u * kBN < fb_hi; };
+    auto needs_exact = [&](int u) { return u * kBN >= fb_lo; };
     auto request_k = [&](int u, int par) __attribute__((always_inline)) {
-        if (needs_c(u) && (kSlotsC == 2 || u == u0)) copy_k(s_kc(par), kc, p.kc.sn, u * kBN);
-        if (needs_a(u)) copy_k(s_ka(par), ka, p.ka.sn, u * kBN);
+        if (needs_far(u)) copy_k(s_kc(par), kc, p.kc.sn, u * kBN);
+        if (needs_exact(u)) copy_k(s_ka(par), ka, p.ka.sn, u * kBN);
     };
-    auto wave_reads_c = [&](int u) { return KIND == kVq ? u * kBN < fb_w : (KIND == kRerope && u * kBN <= edge_w); };
 
     // the first tiles are requested before anything else of the pass: their latency covers the query loads
-    request_k(u0, 0);
-    copy_v(s_v(0), u0 * kBN);
-    if (u0 + 1 < n_iter) request_k(u0 + 1, 1);
+    request_k(0, 0);
+    copy_v(s_v(0), 0);
+    if (n_iter > 1) request_k(1, 1);
 
     flash2::Wave<Tag, D> w;
     w.init();
-    {
-        // kRerope: a wave that meets second-pair keys starts with the second query and changes over at its edge tile
-        const uint16_t* src = (KIND == kRerope && edge_w >= 0) ? q2_src : q_src;
-        const int64_t sn_q = (KIND == kRerope && edge_w >= 0) ? p.q2.sn : p.q.sn;
-        flash::load_q<Tag, D>(w.q[0], src, sn_q, row0, p.N, lane);
-        flash::load_q<Tag, D>(w.q[1], src, sn_q, row0 + 32, p.N, lane);
-        flash2::prescale_q<Tag, D>(w.q[0], p.scale_log2e);
-        flash2::prescale_q<Tag, D>(w.q[1], p.scale_log2e);
-    }
+    flash::load_q<Tag, D>(w.q[0], q_src, p.q.sn, row0, p.N, lane);
+    flash::load_q<Tag, D>(w.q[1], q_src, p.q.sn, row0 + 32, p.N, lane);
+    flash2::prescale_q<Tag, D>(w.q[0], p.scale_log2e);
+    flash2::prescale_q<Tag, D>(w.q[1], p.scale_log2e);
 
     Scores s_even, s_odd;
     typename Pipe::Frags kf, vf;
     float mx[2] = {-INFINITY, -INFINITY};
 
-    // masks of tile u for this wave: causal diagonal, lower window edge and end of the sequence; a tile past the
-    // wave's last row (or past the last tile) ends up fully masked
+    // masks of tile u for this wave: causal diagonal and end of the sequence; a tile past the wave's last row (or
+    // past the last tile) ends up fully masked
     auto mask_tile = [&](Scores& sn, int u) __attribute__((always_inline)) {
         const int n0 = u * kBN;
-        const bool causal = KIND != kVq || p.causal;
-        const int lo_last = lo_w + ((KIND == kWindow && p.strict) ? flash2::kWaveRows - 1 : 0);  // of the wave's last row
-        const bool whole = (n0 + kBN <= p.N) && (!causal || n0 + kBN - 1 <= row0) && u < n_iter &&
-                           (KIND == kVq || n0 >= lo_last);
+        const bool whole = (n0 + kBN <= p.N) && (!p.causal || n0 + kBN - 1 <= row0) && u < n_iter;
         if (whole) return;  // (wave-uniform)
         flash2::mfma_settle(sn);  // the scores below were produced by the last MFMAs
         const int lane_o = flash2::opaque_lane(lane);  // keeps the predicates inside this branch
@@ -206,54 +170,32 @@ __global__ __launch_bounds__(64 * waves_of<KIND>(), 1) void prefill_pipe_kernel(
 #pragma unroll
         for (int qb = 0; qb < 2; ++qb) {
             const int i = row0 + qb * 32 + (lane_o & 31);
-            const int lim = causal ? min(j_hi, i + 1) : j_hi;  // keys lo <= j < lim are visible
-            const int lo = KIND == kVq ? 0 : lo_w + ((KIND == kWindow && p.strict) ? i - row0 : 0);
+            const int lim = p.causal ? min(j_hi, i + 1) : j_hi;  // keys j < lim are visible
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int j = n0 + kb * 32 + flash::key_of_reg(r, half);
-                    const bool vis = KIND == kVq ? j < lim : (j < lim && j >= lo);
-                    sn.s[qb][kb][r] = vis ? sn.s[qb][kb][r] : -INFINITY;
+                    sn.s[qb][kb][r] = j < lim ? sn.s[qb][kb][r] : -INFINITY;
                 }
         }
     };
-    // after the scores of tile u: masks, and at the wave's ReRoPE edge tile the change-over to the first pair (the
-    // scores so far are q2.k2; keys with i - j <= W take q1.k1, and q1 serves every later tile)
-    auto finish_scores = [&](Scores& sn, int u, int par) __attribute__((always_inline)) {
-        mask_tile(sn, u);
-        if constexpr (KIND == kRerope) {
-            if (u * kBN == edge_w) {  // (wave-uniform; every key of this tile is visible to every row of the wave)
-                flash::load_q<Tag, D>(w.q[0], q_src, p.q.sn, row0, p.N, lane);
-                flash::load_q<Tag, D>(w.q[1], q_src, p.q.sn, row0 + 32, p.N, lane);
-                flash2::prescale_q<Tag, D>(w.q[0], p.scale_log2e);
-                flash2::prescale_q<Tag, D>(w.q[1], p.scale_log2e);
-                const int lane_o = flash2::opaque_lane(lane);
-                const int half = lane_o >> 5, n = lane_o & 31;
-                Pipe::second_pair(w, sn, s_ka(par), lane, [&](int qb, int kb, int r) {
-                    // i - j <= W  with  i = row0 + qb*32 + n,  j = edge_w + kb*32 + key:  qb*32 + n <= kb*32 + key
-                    return qb * 32 + n <= kb * 32 + flash::key_of_reg(r, half);
-                });
-            }
-        }
-    };
-    auto k_tile_of_wave = [&](int u, int par) { return wave_reads_c(u) ? s_kc(par) : s_ka(par); };
+    auto k_tile_of_wave = [&](int u, int par) { return (u * kBN < fb_w) ? s_kc(par) : s_ka(par); };
     const typename Pipe::TileRequest no_req{nullptr, 0};
 
-    // first tile: scores, masks, row maxima (nothing to overlap with yet).  Buffer parity follows u - u0.
+    // first tile: scores, masks, row maxima (nothing to overlap with yet)
     flash::wait_tile_loads();
     __syncthreads();
-    Pipe::k_head(kf, k_tile_of_wave(u0, 0), lane);
+    Pipe::k_head(kf, k_tile_of_wave(0, 0), lane);
     Pipe::template score_phase<true, false, false, false>(w, s_even, kf, s_odd, vf, 0u, lane, kd_c, no_req, vd, no_req);
-    finish_scores(s_even, u0, 0);
+    mask_tile(s_even, 0);
     Pipe::template pv_phase<false, true>(w, vf, s_odd, s_even, mx);
 
     // Row addresses of this wave's share of the tiles the main loop requests next: K tile u + 2, V tile u + 1.
     const int64_t kc_step = (int64_t)kBN * p.kc.sn * 2, ka_step = (int64_t)kBN * p.ka.sn * 2, v_step = (int64_t)kBN * p.v.sn * 2;
-    const int r2 = (u0 + 2) * kBN + wave * KDma::kRowsPerWave;
-    const char* kc_rows = reinterpret_cast<const char*>(kc + (int64_t)r2 * p.kc.sn);
-    const char* ka_rows = reinterpret_cast<const char*>(ka + (int64_t)r2 * p.ka.sn);
-    const char* v_rows = reinterpret_cast<const char*>(v_src + (int64_t)(r2 - kBN) * p.v.sn);
+    const char* kc_rows = reinterpret_cast<const char*>(kc + (int64_t)(2 * kBN + wave * KDma::kRowsPerWave) * p.kc.sn);
+    const char* ka_rows = reinterpret_cast<const char*>(ka + (int64_t)(2 * kBN + wave * KDma::kRowsPerWave) * p.ka.sn);
+    const char* v_rows = reinterpret_cast<const char*>(v_src + (int64_t)(kBN + wave * VDma::kRowsPerWave) * p.v.sn);
     // Iteration u finishes tile u (exponentials, P.V) and prepares tile u + 1 (scores, masks, row maxima); K(u+1) and
     // V(u) were requested one iteration earlier and sit in the buffers of parity u + 1 and u.  It requests K(u+2) and
     // V(u+1): whole tiles ride on the score MFMAs (kRide), anything else goes out as a block in front of them.
@@ -264,30 +206,19 @@ __global__ __launch_bounds__(64 * waves_of<KIND>(), 1) void prefill_pipe_kernel(
         Scores& sn = par ? s_even : s_odd;
         flash::wait_tile_loads();
         __syncthreads();  // K(u+1) and V(u) are complete; every wave is done with K(u) and V(u-1)
-        if constexpr (kSlotsC == 1) {
-            // the one second-source slot is free now: the tile about to be scored is brought and waited for (once or
-            // twice per query tile; the other workgroup of the CU computes meanwhile)
-            if (needs_c(u + 1)) {  // (workgroup-uniform)
-                copy_k(s_kc(0), kc, p.kc.sn, (u + 1) * kBN);
-                flash::wait_tile_loads();
-                __syncthreads();
-            }
-        }
         Pipe::k_head(kf, k_tile_of_wave(u + 1, par + 1), lane);
         typename Pipe::TileRequest kr = no_req, vr = no_req;
         KDma kd = kd_c;
         if constexpr (kRide) {
             const int n2 = (u + 2) * kBN;
-            // the source every wave may need rides; where some waves need the other one too, it follows as a block
-            const bool ride_c = KIND == kVq && needs_c(u + 2);
-            kr.rows = ride_c ? kc_rows : ka_rows;
-            kr.lds = KDma::lds_of_wave(ride_c ? s_kc(par) : s_ka(par), wave);
+            const bool far = needs_far(u + 2);
+            kr.rows = far ? kc_rows : ka_rows;
+            kr.lds = KDma::lds_of_wave(far ? s_kc(par) : s_ka(par), wave);
 #pragma unroll
-            for (int i = 0; i < KDma::kInstr; ++i) kd.off[i] = ride_c ? kd_c.off[i] : kd_a.off[i];
+            for (int i = 0; i < KDma::kInstr; ++i) kd.off[i] = far ? kd_c.off[i] : kd_a.off[i];
             vr.rows = v_rows;
             vr.lds = VDma::lds_of_wave(s_v(par + 1), wave);
-            if (KIND == kVq && ride_c && needs_a(u + 2)) copy_k(s_ka(par), ka, p.ka.sn, n2);
-            if (KIND == kRerope && kSlotsC == 2 && needs_c(u + 2)) copy_k(s_kc(par), kc, p.kc.sn, n2);
+            if (far && needs_exact(u + 2)) copy_k(s_ka(par), ka, p.ka.sn, n2);  // boundary tile: both sources
             kc_rows += kc_step, ka_rows += ka_step, v_rows += v_step;
         } else {
             if (u + 2 < n_iter) request_k(u + 2, par);
@@ -295,12 +226,12 @@ __global__ __launch_bounds__(64 * waves_of<KIND>(), 1) void prefill_pipe_kernel(
         }
         Pipe::update_max(w, mx, sc);
         Pipe::template score_phase<true, true, true, kRide>(w, sn, kf, sc, vf, s_v(par), lane, kd, kr, vd, vr);
-        finish_scores(sn, u + 1, par + 1);
+        mask_tile(sn, u + 1);
         mx[0] = mx[1] = -INFINITY;
         Pipe::template pv_phase<true, true>(w, vf, sc, sn, mx);
     };
     // main loop: pairs of iterations whose requests are whole tiles; then the last few, which may run over the end
-    int u = u0;
+    int u = 0;
     for (; u + 3 < n_whole; u += 2) {
         iteration(std::false_type{}, std::true_type{}, u);
         iteration(std::true_type{}, std::true_type{}, u + 1);
@@ -313,7 +244,7 @@ __global__ __launch_bounds__(64 * waves_of<KIND>(), 1) void prefill_pipe_kernel(
     // the output rows leave through LDS (every wave its own part of the tile buffers) once no wave reads tiles any more
     Pipe::settle_o(w);
     __syncthreads();
-    static_assert((size_t)NW * Pipe::kStoreBytes <= lds_bytes<D, KIND>(), "staging area exceeds the tile buffers");
+    static_assert((size_t)4 * Pipe::kStoreBytes <= lds_bytes<D>(), "staging area exceeds the tile buffers");
     Pipe::store(w, p.out + b * p.o_sb + h * p.o_sh, p.o_sn, p.lse ? p.lse + (int64_t)bh * p.N : nullptr, row0, p.N,
                 lane, smem + wave * Pipe::kStoreBytes);
     }
@@ -321,7 +252,7 @@ __global__ __launch_bounds__(64 * waves_of<KIND>(), 1) void prefill_pipe_kernel(
 
 // ---------------------------------------------------------------------------------------------------------------
 // Sliding-window kinds (kWindow, kRerope): 128-row query tiles (2 waves), two workgroups per CU, and every workgroup
-// walks a run of consecutive query tiles of one (batch, head).  A query tile meets only (W + 128) / 64 key tiles, so
+// walks several query tiles of one (batch, head).  A query tile meets only (W + 128) / 64 key tiles, so
 // what surrounds its key loop weighs as much as the loop: a cold start (first tiles and queries from HBM), the
 // drained software pipeline, the output rows, the launch of the next workgroup.  Walking a run removes the launches
 // and lets the LAST iteration of a query tile -- which has no next key tile to score -- bring the first tiles and the
@@ -594,7 +525,7 @@ __global__ __launch_bounds__(128, 1) void window_pipe_kernel(Params p) {
     }
 }
 
-template <typename Tag, int D, int KIND>
+template <typename Tag, int D>
 int launch(Params p, int B, hipStream_t stream) {
     // more than the 64 KB of LDS a launch gets by default: raised once per device and instantiation
     static std::mutex mu;
@@ -605,21 +536,19 @@ int launch(Params p, int B, hipStream_t stream) {
     {
         std::lock_guard<std::mutex> lock(mu);
         if (!raised[dev]) {
-            if (hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_pipe_kernel<Tag, D, KIND>),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes<D, KIND>()) != hipSuccess) {
+            if (hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_pipe_kernel<Tag, D>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes<D>()) != hipSuccess) {
                 (void)hipGetLastError();
                 return VQA_ERR_LAUNCH_FAILED;
             }
             raised[dev] = true;
         }
     }
-    constexpr int kBM = waves_of<KIND>() * flash2::kWaveRows;
     const int n_tiles = (p.N + kBM - 1) / kBM;
     // causal work grows with the query tile: late and early tiles are paired once there are enough workgroups
-    p.pair_tiles = (KIND == kVq && p.causal && (int64_t)(n_tiles / 2) * B * p.H >= 512) ? 1 : 0;
+    p.pair_tiles = (p.causal && (int64_t)(n_tiles / 2) * B * p.H >= 512) ? 1 : 0;
     const dim3 grid(p.pair_tiles ? (n_tiles + 1) / 2 : n_tiles, B * p.H);
-    constexpr size_t kLds = lds_bytes<D, KIND>();
-    hipLaunchKernelGGL((prefill_pipe_kernel<Tag, D, KIND>), grid, dim3(kBM), kLds, stream, p);
+    hipLaunchKernelGGL((prefill_pipe_kernel<Tag, D>), grid, dim3(flash2::kThreads), lds_bytes<D>(), stream, p);
     return launch_status();
 }
 
@@ -642,11 +571,14 @@ int launch_window(Params p, int B, hipStream_t stream) {
             raised[dev] = true;
         }
     }
-    // runs of consecutive query tiles per workgroup: as long as possible while two rounds of workgroups remain for
-    // the 512 places (256 CUs x 2) of the chip
+    // Query tiles per workgroup.  Short windows: one workgroup per place of the chip (256 CUs x 2), which walks all
+    // its tiles -- no second launch round, every start but the first overlapped (W = 512 at 16k tokens: 524 us against
+    // 538 with two rounds and 555 with four).  Long windows: two rounds, which balance better (W = 4096: 1 645 us
+    // against 1 752).
     const int n_tiles = (p.N + 127) / 128;
     const int64_t total = (int64_t)n_tiles * B * p.H;
-    p.tiles_per_wg = (int)std::max<int64_t>(1, std::min<int64_t>(16, total / 1024));
+    const int64_t places = (p.window + 128) / kBN <= 20 ? 512 : 1024;
+    p.tiles_per_wg = (int)std::max<int64_t>(1, std::min<int64_t>(32, total / places));
     const dim3 grid((n_tiles + p.tiles_per_wg - 1) / p.tiles_per_wg, B * p.H);
     hipLaunchKernelGGL((window_pipe_kernel<Tag, D, KIND>), grid, dim3(128), kLds, stream, p);
     return launch_status();
@@ -655,8 +587,8 @@ int launch_window(Params p, int B, hipStream_t stream) {
 template <typename Tag, int KIND>
 int launch_d(const Params& p, int B, int D, hipStream_t stream) {
     if constexpr (KIND == kVq) {
-        if (D == 64) return launch<Tag, 64, KIND>(p, B, stream);
-        if (D == 128) return launch<Tag, 128, KIND>(p, B, stream);
+        if (D == 64) return launch<Tag, 64>(p, B, stream);
+        if (D == 128) return launch<Tag, 128>(p, B, stream);
     } else {
         if (D == 64) return launch_window<Tag, 64, KIND>(p, B, stream);
         if (D == 128) return launch_window<Tag, 128, KIND>(p, B, stream);

@@ -532,13 +532,13 @@ int local_attn(const void* q1, const void* q2, const void* k1, const void* k2, c
         return prefill_pipe_run<Tag>(p.qa, p.ka, p.ka, p.v, p.out, p.o_sb, p.o_sh, p.o_sn, p.lse, B, H, N, D, cover, 1,
                                      false, p.scale_log2e, stream);
     }
-    // Sliding windows: the pipelined core (128-row query tiles, two workgroups per CU) where it is the faster one.  A
-    // query tile meets (W + 128) / 64 key tiles, and a workgroup's start and end (cold first tiles and queries, output
-    // rows) are not overlapped with anything on its SIMDs, so it needs long windows: measured over batch x heads
-    // 8 - 128, 2k - 32k tokens, windows 128 - 2048 it takes 0.77 - 0.99 of the tiled kernel's time from W = 1024 on
-    // with at least 2048 workgroups, 1.03 - 1.47 below.
-    if (mode <= kLocalRerope && window_pipe_applies(window, N) && (D == 64 || D == 128) && window >= 128 &&
-        (int64_t)((N + 127) / 128) * B * H >= 1) {
+    // Sliding windows: the pipelined core (vqa_prefill_pipe.hip: 128-row query tiles, two workgroups per CU, every
+    // workgroup walking several query tiles) where it is the faster one.  Measured against the tiled kernel over
+    // batch x heads 4 - 128, 2k - 32k tokens, head dims 64 and 128, the three window modes: 0.73 - 0.97 of its time
+    // from W = 512 on (0.84 - 0.88 at W = 512, 16k tokens, 64 heads; 0.78 - 0.81 at W = 2048), level at W = 128 and on
+    // grids of under a thousand query tiles.  The window must be a multiple of 128 and the length one of 64.
+    if (mode <= kLocalRerope && window_pipe_applies(window, N) && (D == 64 || D == 128) && window >= 512 &&
+        (int64_t)((N + 127) / 128) * B * H >= 1024) {
         const int rc = validate(p, B, D);
         if (rc != VQA_OK) return rc;
         return window_pipe_run<Tag>(p.qa, p.qb, p.ka, p.kb, p.v, p.out, p.o_sb, p.o_sh, p.o_sn, p.lse, B, H, N, D,
