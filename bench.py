@@ -22,7 +22,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
 # FETCH_SIZE / WRITE_SIZE scaled by a 1 GiB copy in the same run), not something this script can observe; the figure
 # and the file that documents the run that produced it travel together
 DECODE_MAIN_KERNEL_TRAFFIC = {
-    "bytes": 4_366_794_000,
+    "bytes": 4_364_264_000,
     "source": "profiles/decode_main_kernel_c2_b16_h32_n32768.md (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE; "
               "not measured by this run)",
 }
@@ -129,9 +129,9 @@ def prefill_extra(dev, steps=60, warmup=60, cpu=True):
         "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
                      "duration_covers": "whole call: key reconstruction kernel + fused window/far attention kernel",
-                     # attention kernel 369.7 MB fetched + 67.1 MB written, reconstruction 67.1 MB fetched + 67.1 written
-                     "traffic": 369_738_000 + 67_109_000 + 67_080_000 + 67_109_000,
-                     "traffic_source": "profiles/window_kernel_vq_prefill_c3_h32_n8192_w1024.md (rocprofv3 --pmc "
+                     # attention kernel 360.2 MB fetched + 67.1 MB written, reconstruction 66.0 MB fetched + 57.7 written
+                     "traffic": 360_241_000 + 67_109_000 + 66_003_000 + 57_676_000,
+                     "traffic_source": "profiles/prefill_pipe_kernel_vq_prefill_c3_h32_n8192_w1024.md (rocprofv3 --pmc "
                                        "FETCH_SIZE, then WRITE_SIZE; not measured by this run)"},
     }
     if cpu:
@@ -182,8 +182,8 @@ def local_rerope_extra(dev, steps=60, warmup=60, cpu=True):
         "mfma_frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
         "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4), "duration_covers": "the one window kernel",
-                     "traffic": 2_176_082_000 + 270_157_000,
-                     "traffic_source": "profiles/window_kernel_local_rerope_c4_b2_h32_n16384_w512.md (rocprofv3 --pmc "
+                     "traffic": 1_665_140_000 + 268_468_000,
+                     "traffic_source": "profiles/window_pipe_kernel_local_rerope_c4_b2_h32_n16384_w512.md (rocprofv3 --pmc "
                                        "FETCH_SIZE, then WRITE_SIZE; not measured by this run)"},
     }
     if cpu:
@@ -211,7 +211,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-prefill", action="store_true", help="skip the (untimed-region) prefill measurement")
     ap.add_argument("--no-c5", action="store_true", help="skip the (untimed-region) 32-layer decode harness")
-    ap.add_argument("--c5-steps", type=int, default=16)
+    ap.add_argument("--c5-steps", type=int, default=128, help="decode steps of the 32-layer harness (the configured 128)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="before the timed region, run one plain 1 GiB device copy (reference dispatch of known "
                          "size for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE counters)")
@@ -310,11 +310,11 @@ def main():
         c5 = decode_harness.run(steps=args.c5_steps, warmup=4)
         c5["roofline"] = {"bound": "hbm", "achieved": c5["attention_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                           "frac": c5["attention_hbm_frac"],
-                          "duration_covers": "HIP events around the attention calls of all 32 layers (clamped query, "
-                                             "lookup table, streaming kernel, merge), per decode step, launches "
+                          "duration_covers": "HIP events around the attention calls of all 32 layers (lookup table "
+                                             "with the clamped rotary of the query, streaming kernel, merge), per decode step, launches "
                                              "queued ahead of the GPU",
-                          # streaming kernel 2 187.4 MB per layer (fetch + write counters), table and merge kernels 9.8 MB
-                          "traffic": 32 * (2_187_400_000 + 9_800_000),
+                          # streaming kernel 2 187.5 MB per layer (fetch + write counters), table and merge kernels 9.9 MB
+                          "traffic": 32 * (2_187_461_000 + 9_932_000),
                           "traffic_source": "profiles/decode_harness_c5_b4_n65536.md (rocprofv3 --pmc FETCH_SIZE, then "
                                             "WRITE_SIZE; not measured by this run)"}
         result["c5"] = c5
