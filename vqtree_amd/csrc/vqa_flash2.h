@@ -505,22 +505,30 @@ struct Pipe {
 
     // Second operand pair of a tile (ReRoPE window edge): where take(qb, kb, r) holds, the score of `sn` is replaced by
     // -m + K tile (lds_k) . q^T with the wave's CURRENT query fragments.  One accumulation chain at a time with a
-    // 16-register temporary; nothing is overlapped with it (it runs once per query tile and wave).
+    // 16-register temporary; the chain's K fragments go through the (idle) fragment ring kf, six ahead, so that the
+    // chain waits for LDS once and not eight times.  Nothing else is overlapped with it (it runs once per query tile
+    // and wave).
     template <typename Take>
-    static __device__ __forceinline__ void second_pair(Wave<Tag, D>& w, Scores& sn, uint32_t lds_k, int lane,
+    static __device__ __forceinline__ void second_pair(Wave<Tag, D>& w, Scores& sn, uint32_t lds_k, int lane, Frags& kf,
                                                        Take take) {
         const uint32_t base = frag_base(lds_k, opaque_lane(lane));
+        constexpr int kBuf = 2 * kRingPairs;
+        constexpr int kPre = KS < kBuf ? KS : kBuf;
         static_for<4>([&](auto C) {
             constexpr int qb = decltype(C)::value / 2, kb = decltype(C)::value % 2;
             f32x16_t t;
+            static_for<kPre>([&](auto I) { kf.f[decltype(I)::value] = frag(base, kb, decltype(I)::value); });
             static_for<KS>([&](auto KK) {
                 constexpr int kk = decltype(KK)::value;
-                const u32x4_t a = __builtin_bit_cast(u32x4_t, frag(base, kb, kk));
+                const u32x4_t a = __builtin_bit_cast(u32x4_t, kf.f[kk % kBuf]);
                 const u32x4_t bq = __builtin_bit_cast(u32x4_t, w.q[qb].f[kk]);
                 if constexpr (kk == 0)
                     Mai<Tag>::score_first(t, a, bq, w.negm[qb]);
                 else
                     Mai<Tag>::score(t, a, bq);
+                // the buffer of the fragment used one step ago takes the fragment kBuf - 1 steps ahead
+                if constexpr (kk >= 1 && kk - 1 + kBuf < KS) kf.f[(kk - 1) % kBuf] = frag(base, kb, kk - 1 + kBuf);
+                __builtin_amdgcn_sched_barrier(0);
             });
             mfma_settle(t);
 #pragma unroll

@@ -425,7 +425,7 @@ __global__ __launch_bounds__(128, 1) void window_pipe_kernel(Params p) {
                 flash2::prescale_q<Tag, D>(w.q[1], p.scale_log2e);
                 const int lane_o = flash2::opaque_lane(lane);
                 const int half = lane_o >> 5, n = lane_o & 31;
-                Pipe::second_pair(w, sn, s_ka(par), lane, [&](int qb, int kb, int r) {
+                Pipe::second_pair(w, sn, s_ka(par), lane, kf, [&](int qb, int kb, int r) {
                     // i - j <= W  with  i = row0 + qb*32 + n,  j = edge_w + kb*32 + key:  qb*32 + n <= kb*32 + key
                     return qb * 32 + n <= kb * 32 + flash::key_of_reg(r, half);
                 });
