@@ -2,7 +2,8 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-One step = one seqlen_q = 1 VQ-attention call (lookup table + streaming kernel + split merge) over the decode
+One step = one seqlen_q = 1 VQ-attention call (lookup table + streaming kernel; a split merge where a (batch, head)
+unit is split, which this workload is not) over the decode
 configuration: batch 16, 32 heads, head_dim 128, 32768 keys, 4 codebooks x 256 codewords, bf16, inputs resident in
 HBM.  Prints ONE JSON line.  `value` is the achieved HBM rate of the whole step: algorithmic bytes (codes + V +
 codebooks + q + out, each touched once) divided by the step time.

@@ -285,7 +285,7 @@ def run(layers=32, hidden=4096, heads=32, head_dim=128, ffn=11008, vocab=32000, 
         "attention_us_per_step_host_paced": round(paced_us, 1),
         "note": "us_per_step is whole-step wall time of the plain Python loop (projections, MLP, key encoder, "
                 "attention), which is host-bound; attention_us_per_step sums HIP-event intervals around the attention "
-                "calls of all layers (clamped query, lookup table, streaming kernel, merge) over "
+                "calls of all layers (lookup table with the clamped rotary of the query, streaming kernel, merge) over "
                 f"{ahead_steps} steps whose launches were queued ahead of the GPU behind a device-side sleep, i.e. GPU "
                 "time without launch gaps; attention_us_per_step_host_paced is the same sum taken in the plain loop",
     }
