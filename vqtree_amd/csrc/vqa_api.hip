@@ -3,7 +3,7 @@
 
 extern "C" {
 
-int vqa_version(void) { return 100; /* 0.1.0 */ }
+int vqa_version(void) { return 110; /* 0.1.1: vqa_decode_roped_*, window kinds of the pipelined core */ }
 
 const char* vqa_strerror(int status) {
     switch (status) {
