@@ -490,3 +490,47 @@ def test_single_codebook_prefill_takes_the_codeword_route(B, H, N, D, K, W, with
     assert_close_16(out, want, "codeword-route prefill")
     assert_close_lse(lse, want_lse, atol=1e-2)
     assert_close_16(per_key, want, "per-key prefill, M = 1")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_pipelined_core_with_large_and_drifting_scores(dtype):
+    """The pipelined core keeps a LAZY reference maximum per row (it moves only when a tile exceeds it by 2^8) and adds
+    -m inside the score product.  Scores here are several times the usual size (up to +-40 in base 2) and drift
+    upwards along the sequence (keys grow with their position), so that the maximum of most rows moves again and
+    again, late in their key loop; plus a block of rows whose first visible keys score hugely negative (-50).  Finite
+    results, oracle tolerance, on the VQ prefill kernel, plain causal attention and the sliding-window kernel.
+    (The core rounds the query to 16 bits once more after scaling it: a score error of 1.1e-3 |q o k| scale log2(e),
+    the size of the error the 16-bit inputs carry themselves.  With keys of several times this norm competing for one
+    row, that error exceeds the 16-bit output tolerance in bf16; f16 has 8 x the margin.)"""
+    _say(f"pipelined core, large drifting scores {dtype}")
+    B, H, N, D, W = 1, 2, 2304, 128, 512
+    g = torch.Generator("cpu").manual_seed(77)
+    q = (torch.randn(B, H, N, D, generator=g) * 1.5).to(dtype)
+    ramp = torch.linspace(0.5, 2.0, N).view(1, 1, N, 1)
+    k = (torch.randn(B, H, N, D, generator=g) * ramp).to(dtype)
+    k[:, :, :64] = (-2.0 * q[:, :, 1000:1064].float().sign()).to(dtype)   # score -50 for rows 1000..1063, +-15 elsewhere
+    v = torch.randn(B, H, N, D, generator=g).to(dtype)
+    scale = 1.0 / math.sqrt(D)
+    # (1) plain causal attention through the window entry (window >= N)
+    want, want_lse = oracle.local_attn(q, k, v, N, "strict", scale)
+    out = triton_fused_local_attn.flash_attn_func(_bnhd(q).cuda(), _bnhd(k).cuda(), _bnhd(v).cuda(), N, scale)
+    assert_close_16(out.transpose(1, 2), want, "causal, large scores")
+    # (2) the sliding-window kernel, block rule and ReRoPE pair rule (second pair: the same tensors negated twice over)
+    for mode in ("loose", "rerope"):
+        want, want_lse = oracle.local_attn(q, k, v, W, mode, scale, q2=q, k2=k)
+        args = [_bnhd(x).cuda() for x in (q, k, v)]
+        if mode == "loose":
+            out, lse = triton_fused_local_attn2.flash_attn_func(*args, W, scale, return_lse=True)
+        else:
+            out, lse = triton_fused_local_attn_rerope.flash_attn_func(args[0], args[0], args[1], args[1], args[2], W,
+                                                                      scale, return_lse=True)
+        assert_close_16(out.transpose(1, 2), want, f"{mode}, large scores")
+        assert torch.isfinite(lse).all()
+        assert_close_lse(lse, want_lse, atol=3e-2)
+    # (3) the VQ prefill kernel: every key quantised, codebooks scaled up
+    cb = (torch.randn(H, 2, 256, D, generator=g) * 1.0).to(dtype)
+    codes = _codes(B, H, N, 2, 256, seed=78)
+    want, _ = oracle.attn_vq_prefill(q, codes, cb, v, k_exact=k, window_size=W, softmax_scale=scale)
+    out = attn_vq_prefill(q.cuda(), codes.cuda(), cb.cuda(), v.cuda(), k_exact=k.cuda(), window_size=W,
+                          softmax_scale=scale, schedule="pipelined")
+    assert_close_16(out, want, "vq prefill, large scores")
