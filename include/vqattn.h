@@ -409,6 +409,20 @@ int vqa_preprocess_f16(const int64_t* ids, const void* v, int64_t* cnt, void* cn
                        void* workspace, size_t workspace_bytes, int B, int H, int N, int D, int C,
                        const int64_t* strides, vqa_stream_t stream);
 
+/* The same preprocessing that also leaves the count state of the whole sequence -- what vqa_count_state_add_* (below)
+ * builds from the same ids and values, bit for bit: state_cnt[b,h,c] = #{j : id_j == c} (int32, [B,H,C] contiguous),
+ * state_vsum[b,h,c,:] = sum of v over those keys in position order (fp32, [B,H,C,D] contiguous, 8-byte aligned).  Both
+ * are overwritten, not accumulated.  The walk over each code's keys ends with these totals anyway, so a prefill that
+ * needs both the count-kernel inputs and the generation-step state gets the state for nothing (a separate fold of
+ * 8192 keys costs ~190 us).  Counterpart in the reference: `update_prefill`, ops/attn_vq.py:89-127. */
+int vqa_preprocess_state_bf16(const int64_t* ids, const void* v, int64_t* cnt, void* cnt_elem, void* v_vq, int64_t* vi,
+                              int32_t* state_cnt, float* state_vsum, void* workspace, size_t workspace_bytes, int B,
+                              int H, int N, int D, int C, const int64_t* strides, vqa_stream_t stream);
+
+int vqa_preprocess_state_f16(const int64_t* ids, const void* v, int64_t* cnt, void* cnt_elem, void* v_vq, int64_t* vi,
+                             int32_t* state_cnt, float* state_vsum, void* workspace, size_t workspace_bytes, int B,
+                             int H, int N, int D, int C, const int64_t* strides, vqa_stream_t stream);
+
 /* ------------------------------------------------------------------------------------------------------------------
  * Rotary position embedding in the model's 16-bit type: out = x * cos[pos] + rotate_half(x) * sin[pos] with
  * rotate_half(x) = cat(-x[D/2:], x[:D/2]); each product and the sum are rounded to the element type, so the result

@@ -122,3 +122,30 @@ def test_generation_with_exact_window_equals_the_last_prefill_row(N):
     st = cache.decode_state[0]
     assert st.length == N + steps and st.base == max(0, (N + steps - 1 - W) // 128 * 128)
     assert int(st.state.cnt.sum()) == B * H * st.base
+
+
+@pytest.mark.parametrize("D,dtype,C,N", [(128, torch.bfloat16, 512, 3000), (64, torch.float16, 128, 777), (128, torch.bfloat16, 1024, 100)])
+def test_preprocessing_leaves_the_count_state(D, dtype, C, N):
+    """`segmented_preprocess(..., state=...)` (vqa_preprocess_state_*): the walk that builds the count-kernel inputs
+    ends with every code's key count and fp32 value sum -- the count state.  It must be the state
+    `vqa_count_state_add_*` builds from the same keys, bit for bit (same order of additions), with ids outside
+    [0, C) clamped by both; and the three regular outputs must not change."""
+    print(f"count state from the preprocessing: D{D} C{C} N{N} {dtype}", flush=True)
+    B, H = 2, 3
+    g = torch.Generator("cpu").manual_seed(61)
+    ids = torch.randint(0, C, (B, H, N), generator=g)
+    ids[:, :, ::11] = C + 5
+    ids[:, :, 1::13] = -2
+    v = _randn(B, H, N, D, seed=62, dtype=dtype)
+    want = CountState(B, H, C, D, "cuda").add(ids.cuda(), v)
+    got = CountState(B, H, C, D, "cuda")
+    cnt, v_vq, vi = A.segmented_preprocess(ids.cuda(), v, C, want_int64_counts=True, state=got)
+    cnt0, v_vq0, vi0 = A.segmented_preprocess(ids.cuda(), v, C, want_int64_counts=True)
+    torch.cuda.synchronize()
+    assert got.n_keys == N == want.n_keys
+    assert torch.equal(got.cnt, want.cnt) and torch.equal(got.vsum, want.vsum)
+    assert torch.equal(cnt, cnt0) and torch.equal(v_vq, v_vq0) and torch.equal(vi, vi0)
+    onehot = torch.nn.functional.one_hot(ids.clamp(0, C - 1), C).double()
+    assert torch.equal(got.cnt.cpu(), onehot.sum(2).to(torch.int32))
+    assert torch.allclose(got.vsum.double().cpu(), torch.einsum("bhtc,bhtd->bhcd", onehot, v.double().cpu()),
+                          atol=2e-3, rtol=1e-5)

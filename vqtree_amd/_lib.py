@@ -64,6 +64,8 @@ SIGNATURES = {
     "vqa_preprocess_workspace_bytes": (c_size_t, [c_int] * 4),
     "vqa_preprocess_bf16": (c_int, [_P] * 7 + [c_size_t] + [c_int] * 5 + [_STRIDES, _P]),
     "vqa_preprocess_f16": (c_int, [_P] * 7 + [c_size_t] + [c_int] * 5 + [_STRIDES, _P]),
+    "vqa_preprocess_state_bf16": (c_int, [_P] * 9 + [c_size_t] + [c_int] * 5 + [_STRIDES, _P]),
+    "vqa_preprocess_state_f16": (c_int, [_P] * 9 + [c_size_t] + [c_int] * 5 + [_STRIDES, _P]),
 }
 
 

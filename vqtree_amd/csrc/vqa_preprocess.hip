@@ -34,6 +34,8 @@ struct Params {
     int32_t* hist;      // [B*H, NB, C]   per-block histograms, then inclusive running counts
     int32_t* start;     // [B*H, C]
     int32_t* order;     // [B*H, N]       key position of every sorted row
+    int32_t* state_cnt; // nullable: [B*H, C]    keys per code over the whole sequence
+    float* state_vsum;  // nullable: [B*H, C, D] fp32 value sum per code over the whole sequence
     int H, N, D, C, NB; // NB = ceil(N / 128)
 };
 
@@ -129,6 +131,8 @@ __global__ __launch_bounds__(kBlock) void scatter_kernel(Params p) {
 
 // One wave per code: running fp32 sum of V over the code's keys in position order.  The sorted positions are
 // fetched 64 at a time (one per lane) and the V rows eight at a time, so only the additions form a dependent chain.
+// The totals the wave ends with are the count state of the sequence (per-code key count and fp32 value sum, what
+// vqa_count_state_add_* would build from the same keys, same order of additions): written out when asked for.
 template <typename Tag>
 __global__ __launch_bounds__(256) void segment_sum_kernel(Params p) {
     const int lane = threadIdx.x & 63;
@@ -168,6 +172,9 @@ __global__ __launch_bounds__(256) void segment_sum_kernel(Params p) {
             }
         }
     }
+    if (p.state_vsum != nullptr && live)
+        *reinterpret_cast<float2*>(p.state_vsum + ((int64_t)bh * p.C + c) * p.D + d) = make_float2(a0, a1);
+    if (p.state_cnt != nullptr && lane == 0) p.state_cnt[(int64_t)bh * p.C + c] = e - s;
 }
 
 inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
@@ -182,14 +189,18 @@ inline size_t workspace_bytes(int B, int H, int N, int C) {
 template <typename Tag>
 int preprocess(const int64_t* ids, const void* v, int64_t* cnt, void* cnt_elem, void* v_vq, int64_t* vi,
                void* workspace, size_t ws_bytes, int B, int H, int N, int D, int C, const int64_t* strides,
-               hipStream_t stream) {
+               hipStream_t stream, int32_t* state_cnt = nullptr, float* state_vsum = nullptr) {
     if (!ids || !v || !v_vq || !workspace || !strides) return VQA_ERR_NULL_POINTER;
     if (!vi && N >= kBlock) return VQA_ERR_NULL_POINTER;  // no block-sampled row exists below 128 keys
     if (B <= 0 || H <= 0 || N <= 0 || C <= 0 || C > kMaxCodes || N / kBlock > 65535) return VQA_ERR_BAD_SHAPE;
     if (D < 2 || D > 128 || (D & 1)) return VQA_ERR_UNSUPPORTED_HEAD_DIM;
     if ((int64_t)B * H > 65535) return VQA_ERR_BAD_ARGUMENT;
     if (ws_bytes < workspace_bytes(B, H, N, C)) return VQA_ERR_WORKSPACE_TOO_SMALL;
+    if ((state_cnt == nullptr) != (state_vsum == nullptr)) return VQA_ERR_NULL_POINTER;
+    if ((uintptr_t)state_vsum & 7) return VQA_ERR_MISALIGNED;
     Params p;
+    p.state_cnt = state_cnt;
+    p.state_vsum = state_vsum;
     p.ids = ids;
     p.id_sb = strides[0], p.id_sh = strides[1], p.id_sn = strides[2];
     p.v = static_cast<const uint16_t*>(v);
@@ -250,6 +261,22 @@ int vqa_preprocess_f16(const int64_t* ids, const void* v, int64_t* cnt, void* cn
                        const int64_t* strides, vqa_stream_t stream) {
     return vqa::prep::preprocess<vqa::f16_tag>(ids, v, cnt, cnt_elem, v_vq, vi, workspace, workspace_bytes, B, H, N, D,
                                                C, strides, stream);
+}
+
+int vqa_preprocess_state_bf16(const int64_t* ids, const void* v, int64_t* cnt, void* cnt_elem, void* v_vq, int64_t* vi,
+                              int32_t* state_cnt, float* state_vsum, void* workspace, size_t workspace_bytes, int B,
+                              int H, int N, int D, int C, const int64_t* strides, vqa_stream_t stream) {
+    if (!state_cnt || !state_vsum) return VQA_ERR_NULL_POINTER;
+    return vqa::prep::preprocess<vqa::bf16_tag>(ids, v, cnt, cnt_elem, v_vq, vi, workspace, workspace_bytes, B, H, N,
+                                                D, C, strides, stream, state_cnt, state_vsum);
+}
+
+int vqa_preprocess_state_f16(const int64_t* ids, const void* v, int64_t* cnt, void* cnt_elem, void* v_vq, int64_t* vi,
+                             int32_t* state_cnt, float* state_vsum, void* workspace, size_t workspace_bytes, int B,
+                             int H, int N, int D, int C, const int64_t* strides, vqa_stream_t stream) {
+    if (!state_cnt || !state_vsum) return VQA_ERR_NULL_POINTER;
+    return vqa::prep::preprocess<vqa::f16_tag>(ids, v, cnt, cnt_elem, v_vq, vi, workspace, workspace_bytes, B, H, N, D,
+                                               C, strides, stream, state_cnt, state_vsum);
 }
 
 }  // extern "C"

@@ -412,11 +412,12 @@ def sort_based_preprocess(vq_key_ids, vq_key_onehot, value_states, block=BLOCK_S
     return cum[:, :, block - 1::block].contiguous(), v_vq.to(dtype), vi[:, :, block - 1::block].contiguous()
 
 
-def segmented_preprocess(vq_key_ids, value_states, n_codes, block=BLOCK_SIZE, want_int64_counts=False):
+def segmented_preprocess(vq_key_ids, value_states, n_codes, block=BLOCK_SIZE, want_int64_counts=False, state=None):
     """Same three tensors as `sort_based_preprocess`, built by the HIP preprocessing kernels (per-block histograms,
     scan, scatter into (code, position) order, one running fp32 sum per code) instead of the one-hot cumulative sum,
     argsort and global prefix sum of ops/attn_vq.py:352-384.  Returns (counts [B,H,N//block,C] in the model dtype, or
-    int64 when `want_int64_counts`; v_vq [B,H,N+1,D]; vi [B,H,N//block,C] int64)."""
+    int64 when `want_int64_counts`; v_vq [B,H,N+1,D]; vi [B,H,N//block,C] int64).  `state` (a fresh
+    `count_state.CountState`): the same pass also leaves the count state of all N keys in it."""
     from .. import _lib
     from ._common import SUFFIX, bhn_strides, ptr
 
@@ -436,12 +437,18 @@ def segmented_preprocess(vq_key_ids, value_states, n_codes, block=BLOCK_SIZE, wa
     ws = torch.empty(lib.vqa_preprocess_workspace_bytes(B, H, N, n_codes), dtype=torch.uint8, device=device)
     strides = _lib.strides_array(*bhn_strides(vq_key_ids), *bhn_strides(value_states), *bhn_strides(cnt),
                                  *bhn_strides(cnt), *bhn_strides(v_vq), *bhn_strides(vi))
+    head = (ptr(vq_key_ids), ptr(value_states), ptr(cnt) if want_int64_counts else None,
+            None if want_int64_counts else ptr(cnt), ptr(v_vq), ptr(vi))
+    tail = (ptr(ws), ws.numel(), B, H, N, D, n_codes, strides, _lib.current_stream(device))
     with torch.cuda.device(device):
-        rc = getattr(lib, "vqa_preprocess_" + SUFFIX[dtype])(
-            ptr(vq_key_ids), ptr(value_states), ptr(cnt) if want_int64_counts else None,
-            None if want_int64_counts else ptr(cnt), ptr(v_vq), ptr(vi), ptr(ws), ws.numel(), B, H, N, D, n_codes,
-            strides, _lib.current_stream(device))
+        if state is None:
+            rc = getattr(lib, "vqa_preprocess_" + SUFFIX[dtype])(*head, *tail)
+        else:
+            assert state.n_keys == 0 and state.cnt.shape == (B, H, n_codes) and state.vsum.shape == (B, H, n_codes, D)
+            rc = getattr(lib, "vqa_preprocess_state_" + SUFFIX[dtype])(*head, ptr(state.cnt), ptr(state.vsum), *tail)
     _lib.check(rc)
+    if state is not None:
+        state.n_keys = N
     return cnt, v_vq, vi
 
 
@@ -453,12 +460,18 @@ def long_prefilling_sort_based_linear(query_states, key_states, value_states, po
 
     B, H, N, D = query_states.shape
     dtype = query_states.dtype
+    from .count_state import CountState
+
     ids = quantize_ids(key_states, cache.codebook)
-    cnt, v_vq, vi = segmented_preprocess(ids, value_states, cache.codebook.shape[1], want_int64_counts=True)
+    # the count state of all keys (what the generation steps of the default mode run on) falls out of the same pass
+    state = None
+    if not cache.generation_exact_window and len(cache.seq_lengths) <= layer_idx:
+        state = CountState(B, H, cache.codebook.shape[1], D, value_states.device)
+    cnt, v_vq, vi = segmented_preprocess(ids, value_states, cache.codebook.shape[1], want_int64_counts=True, state=state)
     q1, k1, q2 = rerope_operands(query_states, key_states, position_ids, cache.window_length, rope_base)
     out = vq_attn_forward(q1, q2, k1, cache.codebook, cnt, key_states, value_states, v_vq, vi,
                           cache.window_length, softmax_scale=1 / math.sqrt(D))
-    _remember(cache, layer_idx, ids, value_states, N, k1, key_states)
+    _remember(cache, layer_idx, ids, value_states, N, k1, key_states, state=state)
     return out.transpose(1, 2).contiguous().flatten(2)
 
 
@@ -477,7 +490,7 @@ def long_prefilling_per_key(query_states, key_states, value_states, position_ids
     return out.transpose(1, 2).contiguous().flatten(2)
 
 
-def _remember(cache, layer_idx, ids, value_states, n_tokens, k1, key_states):
+def _remember(cache, layer_idx, ids, value_states, n_tokens, k1, key_states, state=None):
     """Record a prefill in the cache (what `update_prefill` keeps, ops/attn_vq.py:89-127): the sequence length, so
     that the next seqlen_q == 1 call is recognised as a generation step; the codeword ids; and the state the
     generation steps run on -- the count state over all keys, or, with `generation_exact_window`, the count state
@@ -493,11 +506,12 @@ def _remember(cache, layer_idx, ids, value_states, n_tokens, k1, key_states):
         C = cache.codebook.shape[1]
         code_dtype = torch.uint8 if C <= 256 else torch.int16
         cache.key_codes.append(ids.to(code_dtype).unsqueeze(-1).contiguous())
-        state = CountState(B, H, C, D, value_states.device)
-        if cache.generation_exact_window:
-            state = GenerationWindow(cache.window_length, k1, key_states, value_states, ids, n_tokens, state)
-        else:
-            state.add(ids, value_states)
+        if state is None:  # (else: the preprocessing of the linear prefill has built it)
+            state = CountState(B, H, C, D, value_states.device)
+            if cache.generation_exact_window:
+                state = GenerationWindow(cache.window_length, k1, key_states, value_states, ids, n_tokens, state)
+            else:
+                state.add(ids, value_states)
         cache.decode_state.append(state)
         cache.seq_lengths.append(n_tokens)
 
