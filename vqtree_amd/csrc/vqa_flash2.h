@@ -477,19 +477,25 @@ struct Pipe {
         const bool any0 = mx[0] > ((w.m[0] == -INFINITY) ? -INFINITY : kLazy);
         const bool any1 = mx[1] > ((w.m[1] == -INFINITY) ? -INFINITY : kLazy);
         if (__builtin_amdgcn_ballot_w64(any0 || any1) == 0) return;
-        settle_o(w);  // O was last written by the previous tile's final MFMAs
+        // rows that see their first key have l = O = 0: nothing to rescale.  That is every row at the start of a query
+        // tile, so the first tile of a key loop does not pay for reading and writing all of O.
+        const bool resc0 = any0 && w.m[0] != -INFINITY, resc1 = any1 && w.m[1] != -INFINITY;
+        const bool rescale = __builtin_amdgcn_ballot_w64(resc0 || resc1) != 0;
+        if (rescale) settle_o(w);  // O was last written by the previous tile's final MFMAs
 #pragma unroll
         for (int qb = 0; qb < 2; ++qb) {
             const float rel = join_halves_max(mx[qb]);
             const bool first = w.m[qb] == -INFINITY;
             const bool need = rel > (first ? -INFINITY : kLazy);
             const float delta = need ? rel : 0.f;
-            // a first key: l = O = 0, any finite factor keeps them there (2^-rel may overflow)
-            const float alpha = (need && !first) ? fast_exp2(-delta) : (need ? 0.f : 1.f);
-            w.l[qb][0] *= alpha;
-            w.l[qb][1] *= alpha;
+            if (rescale) {
+                // (a first key among rows that do move: any finite factor keeps l = O = 0; 2^-rel may overflow)
+                const float alpha = (need && !first) ? fast_exp2(-delta) : (need ? 0.f : 1.f);
+                w.l[qb][0] *= alpha;
+                w.l[qb][1] *= alpha;
 #pragma unroll
-            for (int db = 0; db < DB; ++db) rescale_acc(w.o[qb][db], alpha);
+                for (int db = 0; db < DB; ++db) rescale_acc(w.o[qb][db], alpha);
+            }
             const float m_old = first ? 0.f : w.m[qb];
             if (need) w.m[qb] = m_old + delta;
             // (-m as old value minus delta, element by element: written like this the register allocator updates the

@@ -389,27 +389,39 @@ __global__ __launch_bounds__(128, 1) void window_pipe_kernel(Params p) {
     mx[0] = mx[1] = -INFINITY;
     const int row0 = g.row0;
 
-    // masks of tile u for this wave: causal diagonal, lower window edge, tiles past the wave's last row
+    // masks of tile u for this wave: causal diagonal, lower window edge, tiles past the wave's last row.  A tile that
+    // lies wholly above the wave's rows, below its window (block rule: the edge is tile-aligned) or past the last
+    // tile is cleared without a compare; on the diagonal one compare per element (the sequence length is a multiple
+    // of the tile, so no key of a tile below n_iter lies past it); the strict rule adds its per-row lower edge.
     auto mask_tile = [&](Scores& sn, int u) __attribute__((always_inline)) {
         const int n0 = u * kBN;
         const int lo_last = g.lo_w + (p.strict ? flash2::kWaveRows - 1 : 0);  // of the wave's last row
         const bool whole = n0 + kBN - 1 <= row0 && u < g.n_iter && n0 >= lo_last;
         if (whole) return;  // (wave-uniform)
         flash2::mfma_settle(sn);  // the scores below were produced by the last MFMAs
+        const bool none = u >= g.n_iter || n0 > row0 + flash2::kWaveRows - 1 || n0 + kBN - 1 < g.lo_w;
+        if (none) {  // (wave-uniform)
+#pragma unroll
+            for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) sn.s[qb][kb][r] = -INFINITY;
+            return;
+        }
         const int lane_o = flash2::opaque_lane(lane);  // keeps the predicates inside this branch
         const int half = lane_o >> 5;
-        const int j_hi = u < g.n_iter ? p.N : 0;  // no such tile: nothing visible
 #pragma unroll
         for (int qb = 0; qb < 2; ++qb) {
-            const int i = row0 + qb * 32 + (lane_o & 31);
-            const int lim = min(j_hi, i + 1);  // keys lo <= j < lim are visible
-            const int lo = g.lo_w + (p.strict ? i - row0 : 0);
+            const int i_rel = row0 - n0 + qb * 32 + (lane_o & 31);  // query row relative to the tile's first key
+            const int lo_rel = p.strict ? i_rel - p.window : -1;    // keys lo_rel <= j - n0 <= i_rel are visible
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
-                    const int j = n0 + kb * 32 + flash::key_of_reg(r, half);
-                    sn.s[qb][kb][r] = (j < lim && j >= lo) ? sn.s[qb][kb][r] : -INFINITY;
+                    const int j_rel = kb * 32 + flash::key_of_reg(r, half);
+                    const bool vis = p.strict ? (j_rel <= i_rel && j_rel >= lo_rel) : j_rel <= i_rel;
+                    sn.s[qb][kb][r] = vis ? sn.s[qb][kb][r] : -INFINITY;
                 }
         }
     };
