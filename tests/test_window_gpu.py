@@ -177,6 +177,24 @@ def test_rerope_full(causal, N, D, W):
     assert_close_16(out, want, "rerope_full")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,H,N,D,W", [(1, 2, 2304, 128, 512), (2, 1, 2100, 128, 64), (1, 2, 3000, 64, 1024),
+                                        (1, 1, 2049, 128, 2048), (1, 8, 2176, 128, 192)])
+def test_causal_rerope_full_on_the_pipelined_core(B, H, N, D, W, dtype):
+    """Causal full-context ReRoPE of 2048 tokens or more with a window that is a multiple of 64 runs on the 256-row
+    pipelined kernel (second-pair tiles with the second query, a change-over with a second product at each wave's
+    edge tile, first-pair tiles up to the diagonal); ragged lengths and a window that reaches back to key 0 for most
+    rows included.  The non-causal call of the same shape stays on the general kernel; both against the oracle."""
+    _say(f"causal rerope_full on the pipelined core B{B} H{H} N{N} D{D} W{W} {dtype}")
+    q1, q2, k1, k2, v = (_randn(B, H, N, D, seed=130 + s, dtype=dtype) for s in range(5))
+    for causal in (True, False):
+        scale = 1.0 / math.sqrt(D)
+        want, _ = oracle.rerope_full(q1, q2, k1, k2, v, causal, scale, W)
+        out = triton_fused_attn_rerope.attention(q1.cuda(), q2.cuda(), k1.cuda(), k2.cuda(), v.cuda(), causal, scale, W)
+        torch.cuda.synchronize()
+        assert_close_16(out, want, f"rerope_full causal={causal}")
+
+
 # ------------------------------------------------------------------ VQ prefill (additive codes)
 def _codes(B, H, N, M, K=256, seed=0):
     g = torch.Generator("cpu").manual_seed(seed)

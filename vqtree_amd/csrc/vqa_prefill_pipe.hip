@@ -56,8 +56,15 @@ constexpr size_t lds_bytes() {
     return (size_t)Geom<D>::kTileBytes * 6;
 }
 
-template <typename Tag, int D>
+// KIND: kVq, or kRerope = causal full-context ReRoPE (ops/triton_fused_attn_rerope.py:114-167): every key j <= i is
+// visible, scored q1.k1 where i - j < W and q2.k2 elsewhere.  To this kernel that is the VQ prefill with the second
+// keys in the place of the reconstructed ones -- a long run of second-source tiles, then first-source tiles up to
+// the diagonal -- plus what the sliding-window kernel does at a wave's window-edge tile: the wave scores its
+// second-source tiles with the second query, and at the tile the edge crosses it loads the first query, gives the tile
+// a second product and keeps the first query from there on.
+template <typename Tag, int D, int KIND>
 __global__ __launch_bounds__(flash2::kThreads, 1) void prefill_pipe_kernel(Params p) {
+    static_assert(KIND == kVq || KIND == kRerope, "kinds of the 256-row kernel");
     typedef Geom<D> G;
     typedef flash2::Pipe<Tag, D> Pipe;
     typedef typename Pipe::KDma KDma;
@@ -97,6 +104,7 @@ __global__ __launch_bounds__(flash2::kThreads, 1) void prefill_pipe_kernel(Param
     const uint16_t* kc = p.kc.p + b * p.kc.sb + h * p.kc.sh;
     const uint16_t* v_src = p.v.p + b * p.v.sb + h * p.v.sh;
     const uint16_t* q_src = p.q.p + b * p.q.sb + h * p.q.sh;
+    const uint16_t* q2_src = p.q2.p + b * p.q2.sb + h * p.q2.sh;
 
     // whole-tile copies that ride on the score MFMAs: per-lane offsets once per kernel (one set per row stride)
     KDma kd_a, kd_c;
@@ -124,11 +132,15 @@ __global__ __launch_bounds__(flash2::kThreads, 1) void prefill_pipe_kernel(Param
     const int row0 = m0 + wave * flash2::kWaveRows;  // this wave's 64 rows (inside one 128-row block)
     if (pass) __syncthreads();  // the previous query tile's last reads of the LDS buffers are done
 
-    // first exact key of the two 128-row blocks of the workgroup, and of this wave's block
+    // kVq: first exact key of the two 128-row blocks of the workgroup, and of this wave's block.
+    // kRerope: the second pair scores the keys j <= i - W, i.e. whole tiles below the wave's edge tile (the one at
+    // row0 - W) and part of that tile: in the same three variables, the first tile that needs the first source at
+    // all (the first wave's edge tile), the end of the last wave's edge tile, the end of this wave's edge tile.
     const int kNever = 0x7fffffff;
+    const int edge_w = KIND == kRerope ? row0 - p.window : -1;
     const int fb_lo = p.all_far ? kNever : max(0, m0 - p.window);
-    const int fb_hi = p.all_far ? kNever : max(0, m0 + kBlock - p.window);
-    const int fb_w = (wave < 2) ? fb_lo : fb_hi;
+    const int fb_hi = p.all_far ? kNever : max(0, m0 + (KIND == kRerope ? kBM : kBlock) - p.window);
+    const int fb_w = KIND == kRerope ? max(0, edge_w + kBN) : ((wave < 2) ? fb_lo : fb_hi);
     // tiles [0, n_iter): keys up to the last row of the query tile (causal) or all of them
     const int hi_key = p.causal ? min(p.N, m1 + 1) : p.N;
     const int n_iter = (hi_key + kBN - 1) / kBN;
@@ -148,10 +160,16 @@ __global__ __launch_bounds__(flash2::kThreads, 1) void prefill_pipe_kernel(Param
 
     flash2::Wave<Tag, D> w;
     w.init();
-    flash::load_q<Tag, D>(w.q[0], q_src, p.q.sn, row0, p.N, lane);
-    flash::load_q<Tag, D>(w.q[1], q_src, p.q.sn, row0 + 32, p.N, lane);
-    flash2::prescale_q<Tag, D>(w.q[0], p.scale_log2e);
-    flash2::prescale_q<Tag, D>(w.q[1], p.scale_log2e);
+    {
+        // kRerope: a wave that meets second-pair keys starts with the second query
+        const bool second = KIND == kRerope && edge_w >= 0;
+        const uint16_t* src = second ? q2_src : q_src;
+        const int64_t sn_q = second ? p.q2.sn : p.q.sn;
+        flash::load_q<Tag, D>(w.q[0], src, sn_q, row0, p.N, lane);
+        flash::load_q<Tag, D>(w.q[1], src, sn_q, row0 + 32, p.N, lane);
+        flash2::prescale_q<Tag, D>(w.q[0], p.scale_log2e);
+        flash2::prescale_q<Tag, D>(w.q[1], p.scale_log2e);
+    }
 
     Scores s_even, s_odd;
     typename Pipe::Frags kf, vf;
@@ -181,6 +199,25 @@ __global__ __launch_bounds__(flash2::kThreads, 1) void prefill_pipe_kernel(Param
         }
     };
     auto k_tile_of_wave = [&](int u, int par) { return (u * kBN < fb_w) ? s_kc(par) : s_ka(par); };
+    // after the scores of tile u: masks, and (kRerope) at the wave's edge tile the change-over to the first pair: the
+    // scores so far are q2.k2, the keys with i - j < W take q1.k1, and q1 serves every later tile
+    auto finish_scores = [&](Scores& sn, int u, int par) __attribute__((always_inline)) {
+        mask_tile(sn, u);
+        if constexpr (KIND == kRerope) {
+            if (u * kBN == edge_w) {  // (wave-uniform; the tile lies below the diagonal: no mask touched it)
+                flash::load_q<Tag, D>(w.q[0], q_src, p.q.sn, row0, p.N, lane);
+                flash::load_q<Tag, D>(w.q[1], q_src, p.q.sn, row0 + 32, p.N, lane);
+                flash2::prescale_q<Tag, D>(w.q[0], p.scale_log2e);
+                flash2::prescale_q<Tag, D>(w.q[1], p.scale_log2e);
+                const int lane_o = flash2::opaque_lane(lane);
+                const int half = lane_o >> 5, n = lane_o & 31;
+                Pipe::second_pair(w, sn, s_ka(par), lane, kf, [&](int qb, int kb, int r) {
+                    // i - j < W  with  i = row0 + qb*32 + n,  j = edge_w + kb*32 + key:  qb*32 + n < kb*32 + key
+                    return qb * 32 + n < kb * 32 + flash::key_of_reg(r, half);
+                });
+            }
+        }
+    };
     const typename Pipe::TileRequest no_req{nullptr, 0};
 
     // first tile: scores, masks, row maxima (nothing to overlap with yet)
@@ -188,7 +225,7 @@ __global__ __launch_bounds__(flash2::kThreads, 1) void prefill_pipe_kernel(Param
     __syncthreads();
     Pipe::k_head(kf, k_tile_of_wave(0, 0), lane);
     Pipe::template score_phase<true, false, false, false>(w, s_even, kf, s_odd, vf, 0u, lane, kd_c, no_req, vd, no_req);
-    mask_tile(s_even, 0);
+    finish_scores(s_even, 0, 0);
     Pipe::template pv_phase<false, true>(w, vf, s_odd, s_even, mx);
 
     // Row addresses of this wave's share of the tiles the main loop requests next: K tile u + 2, V tile u + 1.
@@ -226,7 +263,7 @@ __global__ __launch_bounds__(flash2::kThreads, 1) void prefill_pipe_kernel(Param
         }
         Pipe::update_max(w, mx, sc);
         Pipe::template score_phase<true, true, true, kRide>(w, sn, kf, sc, vf, s_v(par), lane, kd, kr, vd, vr);
-        mask_tile(sn, u + 1);
+        finish_scores(sn, u + 1, par + 1);
         mx[0] = mx[1] = -INFINITY;
         Pipe::template pv_phase<true, true>(w, vf, sc, sn, mx);
     };
@@ -537,7 +574,7 @@ __global__ __launch_bounds__(128, 1) void window_pipe_kernel(Params p) {
     }
 }
 
-template <typename Tag, int D>
+template <typename Tag, int D, int KIND>
 int launch(Params p, int B, hipStream_t stream) {
     // more than the 64 KB of LDS a launch gets by default: raised once per device and instantiation
     static std::mutex mu;
@@ -548,7 +585,7 @@ int launch(Params p, int B, hipStream_t stream) {
     {
         std::lock_guard<std::mutex> lock(mu);
         if (!raised[dev]) {
-            if (hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_pipe_kernel<Tag, D>),
+            if (hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_pipe_kernel<Tag, D, KIND>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes<D>()) != hipSuccess) {
                 (void)hipGetLastError();
                 return VQA_ERR_LAUNCH_FAILED;
@@ -560,7 +597,7 @@ int launch(Params p, int B, hipStream_t stream) {
     // causal work grows with the query tile: late and early tiles are paired once there are enough workgroups
     p.pair_tiles = (p.causal && (int64_t)(n_tiles / 2) * B * p.H >= 512) ? 1 : 0;
     const dim3 grid(p.pair_tiles ? (n_tiles + 1) / 2 : n_tiles, B * p.H);
-    hipLaunchKernelGGL((prefill_pipe_kernel<Tag, D>), grid, dim3(flash2::kThreads), lds_bytes<D>(), stream, p);
+    hipLaunchKernelGGL((prefill_pipe_kernel<Tag, D, KIND>), grid, dim3(flash2::kThreads), lds_bytes<D>(), stream, p);
     return launch_status();
 }
 
@@ -599,8 +636,8 @@ int launch_window(Params p, int B, hipStream_t stream) {
 template <typename Tag, int KIND>
 int launch_d(const Params& p, int B, int D, hipStream_t stream) {
     if constexpr (KIND == kVq) {
-        if (D == 64) return launch<Tag, 64>(p, B, stream);
-        if (D == 128) return launch<Tag, 128>(p, B, stream);
+        if (D == 64) return launch<Tag, 64, kVq>(p, B, stream);
+        if (D == 128) return launch<Tag, 128, kVq>(p, B, stream);
     } else {
         if (D == 64) return launch_window<Tag, 64, KIND>(p, B, stream);
         if (D == 128) return launch_window<Tag, 128, KIND>(p, B, stream);
@@ -664,6 +701,38 @@ int window_pipe_run(const View& q1, const View& q2, const View& k1, const View& 
     return pipe::launch_d<Tag, pipe::kWindow>(p, B, D, stream);
 }
 
+// causal full-context ReRoPE on the 256-row kernel
+bool rerope_full_pipe_applies(int window, int N, int causal) {
+    return causal && window > 0 && window % pipe::kBN == 0 && window < N;
+}
+
+template <typename Tag>
+int rerope_full_pipe_run(const View& q1, const View& q2, const View& k1, const View& k2, const View& v, uint16_t* out,
+                         int64_t o_sb, int64_t o_sh, int64_t o_sn, float* lse, int B, int H, int N, int D, int window,
+                         float scale_log2e, hipStream_t stream) {
+    pipe::Params p;
+    p.q = q1, p.q2 = q2, p.ka = k1, p.kc = k2, p.v = v;
+    p.out = out;
+    p.o_sb = o_sb, p.o_sh = o_sh, p.o_sn = o_sn;
+    p.lse = lse;
+    p.H = H, p.N = N, p.window = window;
+    p.causal = 1;
+    p.all_far = 0;
+    p.strict = 0;
+    p.pair_tiles = 0;
+    p.tiles_per_wg = 1;
+    p.scale_log2e = scale_log2e;
+    if (D == 64) return pipe::launch<Tag, 64, pipe::kRerope>(p, B, stream);
+    if (D == 128) return pipe::launch<Tag, 128, pipe::kRerope>(p, B, stream);
+    return VQA_ERR_UNSUPPORTED_HEAD_DIM;
+}
+
+template int rerope_full_pipe_run<bf16_tag>(const View&, const View&, const View&, const View&, const View&, uint16_t*,
+                                            int64_t, int64_t, int64_t, float*, int, int, int, int, int, float,
+                                            hipStream_t);
+template int rerope_full_pipe_run<f16_tag>(const View&, const View&, const View&, const View&, const View&, uint16_t*,
+                                           int64_t, int64_t, int64_t, float*, int, int, int, int, int, float,
+                                           hipStream_t);
 template int prefill_pipe_run<bf16_tag>(const View&, const View&, const View&, const View&, uint16_t*, int64_t, int64_t,
                                         int64_t, float*, int, int, int, int, int, int, bool, float, hipStream_t);
 template int prefill_pipe_run<f16_tag>(const View&, const View&, const View&, const View&, uint16_t*, int64_t, int64_t,

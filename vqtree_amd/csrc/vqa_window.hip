@@ -493,6 +493,12 @@ template <typename Tag>
 int prefill_pipe_run(const View& q, const View& ka, const View& kc, const View& v, uint16_t* out, int64_t o_sb,
                      int64_t o_sh, int64_t o_sn, float* lse, int B, int H, int N, int D, int window, int causal,
                      bool all_far, float scale_log2e, hipStream_t stream);
+// causal full-context ReRoPE on the same 256-row kernel (window a multiple of 64)
+bool rerope_full_pipe_applies(int window, int N, int causal);
+template <typename Tag>
+int rerope_full_pipe_run(const View& q1, const View& q2, const View& k1, const View& k2, const View& v, uint16_t* out,
+                         int64_t o_sb, int64_t o_sh, int64_t o_sn, float* lse, int B, int H, int N, int D, int window,
+                         float scale_log2e, hipStream_t stream);
 // the same core for the sliding-window modes (window_rule = Mode 0 / 1 / 2) with a window that is a multiple of 128
 bool window_pipe_applies(int window, int N);
 template <typename Tag>
@@ -543,6 +549,14 @@ int local_attn(const void* q1, const void* q2, const void* k1, const void* k2, c
         if (rc != VQA_OK) return rc;
         return window_pipe_run<Tag>(p.qa, p.qb, p.ka, p.kb, p.v, p.out, p.o_sb, p.o_sh, p.o_sn, p.lse, B, H, N, D,
                                     window, mode, p.scale_log2e, stream);
+    }
+    // Causal full-context ReRoPE on long sequences: the 256-row pipelined kernel (same rule as the VQ prefill).
+    if (mode == kFullRerope && rerope_full_pipe_applies(window, N, causal) && (D == 64 || D == 128) &&
+        N >= kPipeMinTokens) {
+        const int rc = validate(p, B, D);
+        if (rc != VQA_OK) return rc;
+        return rerope_full_pipe_run<Tag>(p.qa, p.qb, p.ka, p.kb, p.v, p.out, p.o_sb, p.o_sh, p.o_sn, p.lse, B, H, N, D,
+                                         window, p.scale_log2e, stream);
     }
     return run<Tag>(p, B, D, mode, stream);
 }
