@@ -130,8 +130,8 @@ def prefill_extra(dev, steps=60, warmup=60, cpu=True):
         "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
                      "duration_covers": "whole call: key reconstruction kernel + fused window/far attention kernel",
-                     # attention kernel 360.2 MB fetched + 67.1 MB written, reconstruction 66.0 MB fetched + 57.7 written
-                     "traffic": 360_241_000 + 67_109_000 + 66_003_000 + 57_676_000,
+                     # attention kernel 356.3 MB fetched + 67.1 MB written, reconstruction 66.0 MB fetched + 57.7 written
+                     "traffic": 356_322_000 + 67_109_000 + 66_003_000 + 57_676_000,
                      "traffic_source": "profiles/prefill_pipe_kernel_vq_prefill_c3_h32_n8192_w1024.md (rocprofv3 --pmc "
                                        "FETCH_SIZE, then WRITE_SIZE; not measured by this run)"},
     }
@@ -183,7 +183,7 @@ def local_rerope_extra(dev, steps=60, warmup=60, cpu=True):
         "mfma_frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
         "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4), "duration_covers": "the one window kernel",
-                     "traffic": 1_665_140_000 + 268_468_000,
+                     "traffic": 1_701_251_000 + 268_443_000,
                      "traffic_source": "profiles/window_pipe_kernel_local_rerope_c4_b2_h32_n16384_w512.md (rocprofv3 --pmc "
                                        "FETCH_SIZE, then WRITE_SIZE; not measured by this run)"},
     }
