@@ -488,6 +488,20 @@ int vqa_count_decode_f16(const void* q, const void* codebook, const int32_t* cnt
                          float* lse, int B, int H, int C, int D, const int64_t* strides, float sm_scale,
                          vqa_stream_t stream);
 
+/*   vqa_count_step: one launch for a whole generation step on the state -- what vqa_count_state_add_* (T = 1),
+ *     vqa_rope_* and vqa_count_decode_* do in three, bit for bit: the new key (codeword id [B,H] int64, clamped; value v
+ *     [B,H,D]) is folded into cnt / vsum, the RAW query is rotated to the position of rope_cos / rope_sin (one [D] row
+ *     each, 4-byte aligned; both NULL: the query comes rotated) and attends over the updated state.
+ *     strides[0..9] = q(b,h) codebook(h,c) out(b,h) id(b,h) v(b,h).  A generation step of the reference's VQ module is
+ *     then two launches (the codeword search for the new key, this), where five separate ones are host-bound. */
+int vqa_count_step_bf16(const void* q, const void* rope_cos, const void* rope_sin, const int64_t* id, const void* v,
+                        const void* codebook, int32_t* cnt, float* vsum, void* out, float* lse, int B, int H, int C,
+                        int D, const int64_t* strides, float sm_scale, vqa_stream_t stream);
+
+int vqa_count_step_f16(const void* q, const void* rope_cos, const void* rope_sin, const int64_t* id, const void* v,
+                       const void* codebook, int32_t* cnt, float* vsum, void* out, float* lse, int B, int H, int C,
+                       int D, const int64_t* strides, float sm_scale, vqa_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

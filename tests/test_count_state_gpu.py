@@ -149,3 +149,34 @@ def test_preprocessing_leaves_the_count_state(D, dtype, C, N):
     assert torch.equal(got.cnt.cpu(), onehot.sum(2).to(torch.int32))
     assert torch.allclose(got.vsum.double().cpu(), torch.einsum("bhtc,bhtd->bhcd", onehot, v.double().cpu()),
                           atol=2e-3, rtol=1e-5)
+
+
+@pytest.mark.parametrize("D,dtype,C", [(128, torch.bfloat16, 512), (64, torch.float16, 128)])
+def test_generation_step_in_one_launch(D, dtype, C):
+    """`count_step` (vqa_count_step_*): the new key folded into the state, the raw query rotated, the count-weighted
+    softmax -- one launch.  Output, lse and the updated state must equal the three-launch sequence (`add`, the rotary
+    kernel, `count_decode`) bit for bit, over several steps in a row, with and without the rotary."""
+    from vqtree_amd.ops.count_state import count_step
+
+    print(f"count state: fused step D{D} C{C} {dtype}", flush=True)
+    B, H, N = 2, 3, 400
+    g = torch.Generator("cpu").manual_seed(71)
+    cb = (_randn(H, C, D, seed=72, dtype=dtype) * 0.5).cuda()
+    ids0 = torch.randint(0, C, (B, H, N), generator=g).cuda()
+    v0 = _randn(B, H, N, D, seed=73, dtype=dtype).cuda()
+    a = CountState(B, H, C, D, "cuda").add(ids0, v0)
+    b = CountState(B, H, C, D, "cuda").add(ids0, v0)
+    cos, sin = A.rope_tables(D, 300, dtype=dtype, device="cuda")
+    pos = 257
+    for step in range(4):
+        q = _randn(B, H, 1, D, seed=80 + step, dtype=dtype).cuda()
+        v = _randn(B, H, 1, D, seed=90 + step, dtype=dtype).cuda()
+        ids = torch.randint(-1, C + 1, (B, H, 1), generator=g).cuda()   # incl. out-of-range ids: clamped
+        rope = (cos[pos], sin[pos]) if step % 2 == 0 else None
+        a.add(ids, v)
+        q_used = A.apply_rope(q, cos, sin, pos) if rope is not None else q
+        want, want_lse = count_decode(q_used, cb, a, return_lse=True)
+        got, got_lse = count_step(q, cb, b, ids, v, rope=rope, return_lse=True)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want) and torch.equal(got_lse, want_lse), f"step {step}"
+        assert torch.equal(a.cnt, b.cnt) and torch.equal(a.vsum, b.vsum) and a.n_keys == b.n_keys

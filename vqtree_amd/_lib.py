@@ -61,6 +61,8 @@ SIGNATURES = {
     "vqa_count_state_add_f16": (c_int, [_P] * 4 + [c_int] * 5 + [_STRIDES, _P]),
     "vqa_count_decode_bf16": (c_int, [_P] * 6 + [c_int] * 4 + [_STRIDES, c_float, _P]),
     "vqa_count_decode_f16": (c_int, [_P] * 6 + [c_int] * 4 + [_STRIDES, c_float, _P]),
+    "vqa_count_step_bf16": (c_int, [_P] * 10 + [c_int] * 4 + [_STRIDES, c_float, _P]),
+    "vqa_count_step_f16": (c_int, [_P] * 10 + [c_int] * 4 + [_STRIDES, c_float, _P]),
     "vqa_preprocess_workspace_bytes": (c_size_t, [c_int] * 4),
     "vqa_preprocess_bf16": (c_int, [_P] * 7 + [c_size_t] + [c_int] * 5 + [_STRIDES, _P]),
     "vqa_preprocess_f16": (c_int, [_P] * 7 + [c_size_t] + [c_int] * 5 + [_STRIDES, _P]),

@@ -108,26 +108,75 @@ __global__ __launch_bounds__(D) void add_kernel(const int64_t* __restrict__ ids,
 // grid B*H, 256 threads.
 constexpr int kDecodeThreads = 256;
 
+// What a generation step adds to the plain decode (all null / unused for vqa_count_decode_*): the new key, folded into
+// the state before the query attends to it, and the rotary of the raw query.
+struct StepArgs {
+    const int64_t* id;      // [B,H] codeword of the new key (clamped into [0, C)); null: plain decode
+    int64_t id_sb, id_sh;
+    const uint16_t* v;      // [B,H,D] value of the new key
+    int64_t v_sb, v_sh;
+    const uint16_t* cos;    // [D] rotary rows of the query's position; null: the query comes rotated
+    const uint16_t* sin;
+};
+
+template <typename Tag>
+__device__ __forceinline__ float rnd_elem(float x) { return Elem<Tag>::round_keep_f32(x); }
+
 template <typename Tag, int D>
 __global__ __launch_bounds__(kDecodeThreads) void decode_kernel(const uint16_t* __restrict__ q,
                                                                 const uint16_t* __restrict__ codebook,
-                                                                const int32_t* __restrict__ cnt,
-                                                                const float* __restrict__ vsum, uint16_t* __restrict__ out,
-                                                                float* __restrict__ lse, int H, int C, int64_t q_sb,
-                                                                int64_t q_sh, int64_t cb_sh, int64_t cb_sc, int64_t o_sb,
-                                                                int64_t o_sh, float scale_log2e) {
+                                                                int32_t* __restrict__ cnt, float* __restrict__ vsum,
+                                                                uint16_t* __restrict__ out, float* __restrict__ lse,
+                                                                int H, int C, int64_t q_sb, int64_t q_sh, int64_t cb_sh,
+                                                                int64_t cb_sc, int64_t o_sb, int64_t o_sh,
+                                                                float scale_log2e, StepArgs step) {
     extern __shared__ float s_e[];  // C scores, then weights exp2(score - max) (0 for codewords with no key)
     __shared__ uint32_t s_q[D / 2];
+    __shared__ uint32_t s_raw[D / 2];
     __shared__ float s_red[kDecodeThreads / kWave];
     __shared__ float s_part[kDecodeThreads / (D / 4)][D];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int bh = blockIdx.x, b = bh / H, h = bh % H;
     const uint16_t* my_q = q + b * q_sb + h * q_sh;
     const uint16_t* my_cb = codebook + h * cb_sh;
-    const int32_t* my_cnt = cnt + (int64_t)bh * C;
-    const float* my_vsum = vsum + (int64_t)bh * C * D;
+    int32_t* my_cnt = cnt + (int64_t)bh * C;
+    float* my_vsum = vsum + (int64_t)bh * C * D;
 
-    if (tid < D / 2) s_q[tid] = reinterpret_cast<const uint32_t*>(my_q)[tid];
+    // A generation step folds the new key in first: cnt[id] += 1, Vsum[id] += v (the fp32 additions of
+    // vqa_count_state_add_*).  One workgroup owns the (batch, head): the barrier below orders these writes before its
+    // own reads of the state.
+    if (step.id != nullptr) {
+        const int64_t raw = step.id[b * step.id_sb + h * step.id_sh];
+        const int id = (int)(raw < 0 ? 0 : (raw >= C ? C - 1 : raw));
+        if (tid < D) my_vsum[(int64_t)id * D + tid] += Elem<Tag>::from_bits(step.v[b * step.v_sb + h * step.v_sh + tid]);
+        if (tid == 0) my_cnt[id] += 1;
+    }
+    if (step.cos == nullptr) {
+        if (tid < D / 2) s_q[tid] = reinterpret_cast<const uint32_t*>(my_q)[tid];
+    } else {
+        // q' = q * cos + rotate_half(q) * sin, every product and the sum rounded to the element type (the bits
+        // vqa_rope_* writes): element pair t of the lower half has its partner pair at t + D/4, and vice versa
+        if (tid < D / 2) s_raw[tid] = reinterpret_cast<const uint32_t*>(my_q)[tid];
+        __syncthreads();
+        if (tid < D / 2) {
+#pragma clang fp contract(off)
+            const bool upper = tid >= D / 4;
+            const uint32_t x = s_raw[tid], xp = s_raw[tid ^ (D / 4)];
+            const uint32_t cw = reinterpret_cast<const uint32_t*>(step.cos)[tid];
+            const uint32_t sw = reinterpret_cast<const uint32_t*>(step.sin)[tid];
+            uint32_t pair = 0;
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                const int sh = 16 * t;
+                const float xv = Elem<Tag>::from_bits((uint16_t)(x >> sh)), pv = Elem<Tag>::from_bits((uint16_t)(xp >> sh));
+                const float cv = Elem<Tag>::from_bits((uint16_t)(cw >> sh)), sv = Elem<Tag>::from_bits((uint16_t)(sw >> sh));
+                const float t0 = rnd_elem<Tag>(xv * cv), t1 = rnd_elem<Tag>(pv * sv);
+                pair |= (uint32_t)Elem<Tag>::to_bits(rnd_elem<Tag>(upper ? t0 + t1 : t0 - t1)) << sh;
+            }
+            s_q[tid] = pair;
+        }
+    }
+    __threadfence_block();
     __syncthreads();
 
     // scores: one codeword per thread; the query is read from LDS at a wave-uniform address (broadcast)
@@ -208,14 +257,16 @@ int add(const int64_t* ids, const void* v, int32_t* cnt, float* vsum, int B, int
 }
 
 template <typename Tag>
-int decode(const void* q, const void* codebook, const int32_t* cnt, const float* vsum, void* out, float* lse, int B,
-           int H, int C, int D, const int64_t* st, float sm_scale, hipStream_t stream) {
+int decode(const void* q, const void* codebook, int32_t* cnt, float* vsum, void* out, float* lse, int B, int H, int C,
+           int D, const int64_t* st, float sm_scale, hipStream_t stream, const StepArgs& step) {
     if (B <= 0 || H <= 0 || C <= 0 || C > VQA_COUNT_STATE_MAX_CODES) return VQA_ERR_BAD_SHAPE;
     if (D != 64 && D != 128) return VQA_ERR_UNSUPPORTED_HEAD_DIM;
     if (!q || !codebook || !cnt || !vsum || !out || !st) return VQA_ERR_NULL_POINTER;
     if (!aligned16(codebook) || (st[2] % 8) || (st[3] % 8) || (reinterpret_cast<uintptr_t>(q) & 3u) || (st[0] % 2) ||
         (st[1] % 2) || !aligned16(vsum))
         return VQA_ERR_MISALIGNED;
+    if ((reinterpret_cast<uintptr_t>(step.cos) | reinterpret_cast<uintptr_t>(step.sin)) & 3u) return VQA_ERR_MISALIGNED;
+    if ((int64_t)B * H > 0x7fffffff) return VQA_ERR_BAD_SHAPE;
     const uint16_t* qp = static_cast<const uint16_t*>(q);
     const uint16_t* cb = static_cast<const uint16_t*>(codebook);
     uint16_t* op = static_cast<uint16_t*>(out);
@@ -223,11 +274,25 @@ int decode(const void* q, const void* codebook, const int32_t* cnt, const float*
     const float scale_log2e = sm_scale * kLog2e;
     if (D == 64)
         hipLaunchKernelGGL((decode_kernel<Tag, 64>), dim3(B * H), dim3(kDecodeThreads), lds, stream, qp, cb, cnt, vsum,
-                           op, lse, H, C, st[0], st[1], st[2], st[3], st[4], st[5], scale_log2e);
+                           op, lse, H, C, st[0], st[1], st[2], st[3], st[4], st[5], scale_log2e, step);
     else
         hipLaunchKernelGGL((decode_kernel<Tag, 128>), dim3(B * H), dim3(kDecodeThreads), lds, stream, qp, cb, cnt, vsum,
-                           op, lse, H, C, st[0], st[1], st[2], st[3], st[4], st[5], scale_log2e);
+                           op, lse, H, C, st[0], st[1], st[2], st[3], st[4], st[5], scale_log2e, step);
     return launch_status();
+}
+
+// strides: q(b,h) codebook(h,c) out(b,h) id(b,h) v(b,h)
+template <typename Tag>
+int step(const void* q, const void* rope_cos, const void* rope_sin, const int64_t* id, const void* v,
+         const void* codebook, int32_t* cnt, float* vsum, void* out, float* lse, int B, int H, int C, int D,
+         const int64_t* st, float sm_scale, hipStream_t stream) {
+    if (!id || !v || !st) return VQA_ERR_NULL_POINTER;
+    if ((rope_cos == nullptr) != (rope_sin == nullptr)) return VQA_ERR_NULL_POINTER;
+    StepArgs a;
+    a.id = id, a.id_sb = st[6], a.id_sh = st[7];
+    a.v = static_cast<const uint16_t*>(v), a.v_sb = st[8], a.v_sh = st[9];
+    a.cos = static_cast<const uint16_t*>(rope_cos), a.sin = static_cast<const uint16_t*>(rope_sin);
+    return decode<Tag>(q, codebook, cnt, vsum, out, lse, B, H, C, D, st, sm_scale, stream, a);
 }
 
 }  // namespace count_state
@@ -246,14 +311,29 @@ int vqa_count_state_add_f16(const int64_t* ids, const void* v, int32_t* cnt, flo
 int vqa_count_decode_bf16(const void* q, const void* codebook, const int32_t* cnt, const float* vsum, void* out,
                           float* lse, int B, int H, int C, int D, const int64_t* strides, float sm_scale,
                           vqa_stream_t stream) {
-    return vqa::count_state::decode<vqa::bf16_tag>(q, codebook, cnt, vsum, out, lse, B, H, C, D, strides, sm_scale,
-                                                   stream);
+    return vqa::count_state::decode<vqa::bf16_tag>(q, codebook, const_cast<int32_t*>(cnt), const_cast<float*>(vsum), out,
+                                                   lse, B, H, C, D, strides, sm_scale, stream,
+                                                   vqa::count_state::StepArgs{});
 }
 int vqa_count_decode_f16(const void* q, const void* codebook, const int32_t* cnt, const float* vsum, void* out,
                          float* lse, int B, int H, int C, int D, const int64_t* strides, float sm_scale,
                          vqa_stream_t stream) {
-    return vqa::count_state::decode<vqa::f16_tag>(q, codebook, cnt, vsum, out, lse, B, H, C, D, strides, sm_scale,
-                                                  stream);
+    return vqa::count_state::decode<vqa::f16_tag>(q, codebook, const_cast<int32_t*>(cnt), const_cast<float*>(vsum), out,
+                                                  lse, B, H, C, D, strides, sm_scale, stream,
+                                                  vqa::count_state::StepArgs{});
+}
+
+int vqa_count_step_bf16(const void* q, const void* rope_cos, const void* rope_sin, const int64_t* id, const void* v,
+                        const void* codebook, int32_t* cnt, float* vsum, void* out, float* lse, int B, int H, int C,
+                        int D, const int64_t* strides, float sm_scale, vqa_stream_t stream) {
+    return vqa::count_state::step<vqa::bf16_tag>(q, rope_cos, rope_sin, id, v, codebook, cnt, vsum, out, lse, B, H, C, D,
+                                                 strides, sm_scale, stream);
+}
+int vqa_count_step_f16(const void* q, const void* rope_cos, const void* rope_sin, const int64_t* id, const void* v,
+                       const void* codebook, int32_t* cnt, float* vsum, void* out, float* lse, int B, int H, int C,
+                       int D, const int64_t* strides, float sm_scale, vqa_stream_t stream) {
+    return vqa::count_state::step<vqa::f16_tag>(q, rope_cos, rope_sin, id, v, codebook, cnt, vsum, out, lse, B, H, C, D,
+                                                strides, sm_scale, stream);
 }
 
 }  // extern "C"

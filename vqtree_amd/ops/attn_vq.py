@@ -572,7 +572,7 @@ def dispatch_attn(query_states, key_states, value_states, position_ids, cache, l
     assert q_len == 1, "Only support prefilling or generation"
     # Generation step on the state the prefill left (the route the reference leaves unimplemented,
     # ops/attn_vq.py:176-223): O(C D) per step, whatever the context length and the codebook size.
-    from .count_state import count_decode
+    from .count_state import count_step
 
     W = cache.window_length
     t = cache.seq_lengths[layer_idx]  # position of the new token
@@ -581,16 +581,17 @@ def dispatch_attn(query_states, key_states, value_states, position_ids, cache, l
     scale = 1 / math.sqrt(D)
     cos, sin = rope_tables(D, max(W + 2, t + 1) if cache.generation_exact_window else W + 2, rope_base,
                            query_states.dtype, query_states.device)
-    q2 = apply_rope(query_states, cos, sin, W + 1)
     if cache.generation_exact_window:
+        q2 = apply_rope(query_states, cos, sin, W + 1)
         # true-position rotary at the positions the caller gives (per batch row; normally all equal to t)
         q1 = apply_rope(query_states, cos, sin, position_ids)
         k1 = apply_rope(key_states, cos, sin, position_ids)
         state.append(k1, key_states, value_states, ids)
         out = state.attend(q1, q2, cache.codebook, scale)
     else:
-        state.add(ids, value_states)
-        out = count_decode(q2, cache.codebook, state, softmax_scale=scale)
+        # one launch: the new key into the state, the clamped rotary of the query, the count-weighted softmax
+        out = count_step(query_states, cache.codebook, state, ids, value_states, rope=(cos[W + 1], sin[W + 1]),
+                         softmax_scale=scale)
     cache.seq_lengths[layer_idx] = t + 1
     if layer_idx == 0:
         cache.seen_tokens += 1

@@ -75,6 +75,37 @@ def count_decode(q, codebook, state, *, softmax_scale=None, return_lse=False):
     return (out, lse) if return_lse else out
 
 
+def count_step(q, codebook, state, ids, v, *, rope=None, softmax_scale=None, return_lse=False):
+    """One generation step on the state in one launch: fold the new key (ids [B,H,1] int64, v [B,H,1,D]) into `state`,
+    rotate the raw query q [B,H,1,D] with `rope = (cos_row, sin_row)` (two [D] rows; None: q comes rotated) and attend
+    over the updated state.  Equal, bit for bit, to `state.add(ids, v)`, `apply_rope(q, ...)`, `count_decode(...)`."""
+    lib = _lib.load()
+    _lib.require_gpu(q, codebook, state.cnt, ids, v)
+    B, H, one, D = q.shape
+    C = codebook.shape[1]
+    assert one == 1 and codebook.shape == (H, C, D) and state.cnt.shape == (B, H, C) and state.vsum.shape[-1] == D
+    assert ids.shape == (B, H, 1) and ids.dtype == torch.int64 and v.shape == (B, H, 1, D)
+    assert q.dtype == codebook.dtype == v.dtype and q.dtype in SUFFIX, "Only support fp16 and bf16"
+    q, v = (t if t.stride(-1) == 1 else t.contiguous() for t in (q, v))
+    codebook = codebook if codebook.stride(-1) == 1 else codebook.contiguous()
+    cos_row = sin_row = None
+    if rope is not None:
+        cos_row, sin_row = (t if t.is_contiguous() else t.contiguous() for t in rope)
+        assert cos_row.shape == sin_row.shape == (D,) and cos_row.dtype == sin_row.dtype == q.dtype
+    softmax_scale = softmax_scale or 1.0 / math.sqrt(D)
+    out = torch.empty((B, H, 1, D), dtype=q.dtype, device=q.device)
+    lse = torch.empty((B, H, 1), dtype=torch.float32, device=q.device) if return_lse else None
+    strides = _lib.strides_array(q.stride(0), q.stride(1), codebook.stride(0), codebook.stride(1), out.stride(0),
+                                 out.stride(1), ids.stride(0), ids.stride(1), v.stride(0), v.stride(1))
+    with torch.cuda.device(q.device):
+        rc = getattr(lib, "vqa_count_step_" + SUFFIX[q.dtype])(
+            ptr(q), ptr(cos_row), ptr(sin_row), ptr(ids), ptr(v), ptr(codebook), ptr(state.cnt), ptr(state.vsum),
+            ptr(out), ptr(lse), B, H, C, D, strides, softmax_scale, _lib.current_stream(q.device))
+    _lib.check(rc)
+    state.n_keys += 1
+    return (out, lse) if return_lse else out
+
+
 def far_boundary(position, window):
     """First key that is NOT replaced by its codeword for the query at `position` (ops/attn_vq.py:283, 311)."""
     return max(0, (position - window) // BLOCK_SIZE * BLOCK_SIZE)
