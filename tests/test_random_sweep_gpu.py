@@ -82,3 +82,44 @@ def test_seeded_random_sweep():
         if not ok:
             failures.append((it, c))
     assert not failures, failures
+
+
+def test_seeded_random_sweep_of_the_pipelined_window_kernels():
+    """The same at the sizes the long-sequence kernels take over: 2k - 6k tokens that are multiples of 64, windows of
+    512 - 3000 keys that are multiples of 128, at least 1024 query tiles; the three window modes and causal
+    full-context ReRoPE, both dtypes and head dims.  Three (batch, head) units per case against the oracle."""
+    rng = random.Random(5)
+    bn = lambda x: x.transpose(1, 2).contiguous()
+    failures = []
+    for it in range(12):
+        D = rng.choice([64, 128, 128])
+        dtype = rng.choice([torch.bfloat16, torch.float16])
+        N = 64 * rng.randint(32, 90)
+        W = 128 * rng.randint(4, max(4, min(24, (N - 64) // 128)))
+        H, B = rng.choice([32, 40, 64]), rng.choice([1, 2])
+        while ((N + 127) // 128) * B * H < 1024:
+            H += 8
+        mode = rng.choice(["strict", "loose", "rerope", "full"])
+        print(f"pipelined sweep {it}: {mode} B{B} H{H} N{N} D{D} W{W} {dtype}", flush=True)
+        g = torch.Generator(device="cuda").manual_seed(100 + it)
+        q, k, v, q2, k2 = (torch.randn(B, H, N, D, generator=g, device="cuda").to(dtype) for _ in range(5))
+        if mode == "strict":
+            out = triton_fused_local_attn.flash_attn_func(bn(q), bn(k), bn(v), W).transpose(1, 2)
+        elif mode == "loose":
+            out = triton_fused_local_attn2.flash_attn_func(bn(q), bn(k), bn(v), W).transpose(1, 2)
+        elif mode == "rerope":
+            out = triton_fused_local_attn_rerope.flash_attn_func(bn(q), bn(q2), bn(k), bn(k2), bn(v), W).transpose(1, 2)
+        else:
+            out = triton_fused_attn_rerope.attention(q, q2, k, k2, v, True, 1.0 / math.sqrt(D), W)
+        torch.cuda.synchronize()
+        for b, h in ((0, 0), (B - 1, H - 1), (0, H // 2)):
+            one = lambda x: x[b:b + 1, h:h + 1].cpu()
+            if mode == "full":
+                want, _ = oracle.rerope_full(one(q), one(q2), one(k), one(k2), one(v), True, 1.0 / math.sqrt(D), W)
+            else:
+                want, _ = oracle.local_attn(one(q), one(k), one(v), W, mode, None, q2=one(q2), k2=one(k2))
+            if not _close(one(out), want):
+                failures.append((it, mode, B, H, N, D, W, dtype, b, h))
+        del q, k, v, q2, k2, out
+        torch.cuda.empty_cache()
+    assert not failures, failures
